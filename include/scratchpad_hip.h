@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define SP_ABI_VERSION 9
+#define SP_ABI_VERSION 10
 #define SP_API __attribute__((visibility("default")))
 
 typedef enum { SP_F32 = 0, SP_F16 = 1, SP_BF16 = 2, SP_FP8_E5M2 = 3 /* KV pool only */ } sp_dtype;
@@ -385,6 +385,101 @@ SP_API int sp_fused_allreduce_add_rmsnorm(void* x, void* residual, const void* w
                                    int hidden, int64_t x_stride, int64_t res_stride, float eps, int dtype,
                                    void* const* regions, int rank, int world, size_t data_bytes,
                                    int64_t timeout_us, void* host_status, void* stream);
+
+/* ================================================================================================================
+ * ABI 10: per-sequence state (token shift, matrix-state recurrence), single-gain norms on an fp32 residual stream,
+ * latent (compressed key/value) attention, mixture of experts.  No reference counterpart: these serve model designs
+ * the reference does not host.
+ *
+ * The requests of a step, as every kernel that touches per-sequence state receives them (SP_SEQ_PARAMS):
+ *   req_pool_indices / seq_lens [batch_size]  int64 (idx64 = 1, eager) or int32 (idx64 = 0, graph replay);
+ *   extend_seq_lens / extend_prefix_lens / extend_start_loc [batch_size] int32 and token_req [num_tokens] int32 (the
+ *   request index of every token row) for a step that brings several tokens per request; all four null for a decode
+ *   step (one row per request, row b = request b, tokens held before = seq_len - 1).  A request with no token held
+ *   before the step starts from the initial state whatever its slot holds, so slots are never cleared on reuse.    */
+#define SP_SEQ_PARAMS                                                                                          \
+  const void *req_pool_indices, const void *seq_lens, const int32_t *extend_seq_lens,                          \
+      const int32_t *extend_prefix_lens, const int32_t *extend_start_loc, const int32_t *token_req, int idx64, \
+      int batch_size
+
+/* rows[t] = (previous token * mul_prev + token * mul_cur) mod buckets, or `buckets` for a sequence's first token;
+ * the previous token of a step's first row is last_token[request slot].  sp_save_last_token stores each request's
+ * last token of this step there (run it after every reader of the step).                                       */
+SP_API int sp_bigram_rows(int32_t* rows, const int64_t* ids, const int64_t* last_token, int64_t num_tokens,
+                          SP_SEQ_PARAMS, int64_t buckets, int64_t mul_prev, int64_t mul_cur, void* stream);
+SP_API int sp_save_last_token(int64_t* last_token, const int64_t* ids, SP_SEQ_PARAMS, void* stream);
+/* state[request slot, :] = x[the request's last row of this step, :]  (fp32) */
+SP_API int sp_save_last_rows(float* state, int64_t state_stride, const float* x, int64_t x_stride, int width,
+                             SP_SEQ_PARAMS, void* stream);
+/* x[t] = (embed[id] + bigram[row]) / rms * gain[0]  (fp32 stream; lo, if given, the same in `dtype`) */
+SP_API int sp_embed_bigram_norm(float* x, void* lo, const void* embed, const void* bigram, const int64_t* ids,
+                                const int32_t* rows, const float* gain, int64_t num_tokens, int width, int64_t x_stride,
+                                int64_t lo_stride, float eps, int dtype, void* stream);
+/* x += y / rms(y) * gain[0] in place on the fp32 stream; lo (optional) = the new x in `dtype`, the type of y */
+SP_API int sp_add_scalar_norm(float* x, void* lo, const void* y, const float* gain, int64_t num_tokens, int width,
+                              int64_t x_stride, int64_t lo_stride, int64_t y_stride, float eps, int dtype, void* stream);
+/* out = x / rms(x) * gain[0], x fp32, out in `dtype` */
+SP_API int sp_scalar_norm(void* out, const float* x, const float* gain, int64_t num_tokens, int width, int64_t x_stride,
+                          int64_t out_stride, float eps, int dtype, void* stream);
+/* out = a N(z) + b N(z^2) + c N(z^3) + e over each row of n values; N divides by the row's root mean square; coef = {a, b, c, e} */
+SP_API int sp_polynorm(void* out, const void* z, const float* coef, int64_t num_tokens, int n, int64_t z_stride,
+                       int64_t out_stride, float eps, int dtype, void* stream);
+/* out[t, h, :] = o[h, t, :] * sigmoid(g[t, h]);  o [heads, T, head_dim], out [T, heads * head_dim] */
+SP_API int sp_gate_heads(void* out, const void* o, const void* g, int64_t num_tokens, int heads, int head_dim,
+                         int64_t g_stride, int dtype, void* stream);
+
+/* out[m, t, :] = x[t] + (x[t - 1] - x[t]) * mu[m]  for m < mixes; x fp32; the row before a step's first row is
+ * shift_state[request slot] (zeros at a sequence's first token); out [mixes, T, width] in `dtype`                */
+SP_API int sp_token_shift(void* out, const float* x, const float* mu, const float* shift_state, int64_t state_stride,
+                          int64_t num_tokens, int width, int mixes, int64_t x_stride, SP_SEQ_PARAMS, int dtype, void* stream);
+/* decay[t, c] = exp(-exp(sum_r w2t[r, c] * tanh(a[t, r]) + w0[c]))  (fp32; a in `dtype`) */
+SP_API int sp_wkv_decay(float* decay, const void* a, const float* w2t, const float* w0, int64_t num_tokens, int channels,
+                        int rank, int64_t a_stride, int dtype, void* stream);
+/* Per (request, head), over the request's rows of this step in order, S [head_dim(key), head_dim(value)] fp32 from
+ * state[request slot] (zeros at a sequence's first token) and back:
+ *   o = (S + diag(u) k v^T)^T r;  S = diag(decay) S + k v^T;  out = o / rms_head(o) * norm_w * silu(g).
+ * r, k, v, g, out: [T, heads * head_dim] in `dtype` with their row strides; decay [T, heads * head_dim] fp32.
+ * head_dim <= 256.                                                                                                */
+SP_API int sp_wkv_recurrence(void* out, const void* r, const void* k, const void* v, const void* g, const float* decay,
+                             const float* u, const float* norm_w, float* state, int64_t state_stride, int heads,
+                             int head_dim, int64_t r_stride, int64_t k_stride, int64_t v_stride, int64_t g_stride,
+                             int64_t out_stride, float eps, SP_SEQ_PARAMS, int dtype, void* stream);
+
+/* In-place rotation of x[t, h, offset .. offset + rot_dim): pairs (2i, 2i + 1), angle = positions[t] * freq[i] in
+ * fp32, cos and sin times mag.                                                                                    */
+SP_API int sp_rotary_interleaved(void* x, const int64_t* positions, const float* freq, float mag, int64_t num_tokens,
+                                 int heads, int rot_dim, int64_t token_stride, int64_t head_stride, int offset, int dtype,
+                                 void* stream);
+/* pool[loc[t]] = [ dkv[t, :rank] / rms * norm_w | dkv[t, rank : rank + rot_dim] with its first rot_dims rotated ] */
+SP_API int sp_latent_kv_store(void* pool, int64_t pool_stride, const void* dkv, int64_t dkv_stride, const float* norm_w,
+                              const int64_t* positions, const float* freq, float mag, const int64_t* loc,
+                              int64_t num_tokens, int rank, int rot_dim, int rot_dims, float eps, int dtype, void* stream);
+/* Causal multi-query attention over pool rows [rank | rot_dim]: score = (q_lat . row[:rank] + q_rot . row[rank:]) * scale,
+ * softmax in fp32, out = sum p * row[:rank].  q_lat, out: [heads, T, rank]; q_rot: x[t * token_stride + h * head_stride + ..].
+ * A token at position p of its request sees the request's positions 0 .. p through req_to_token.  rank <= 1024.  */
+SP_API int sp_latent_attention(void* out, const void* q_lat, const void* q_rot, const void* pool, int64_t pool_stride,
+                               const int32_t* req_to_token, int64_t table_stride, int64_t num_tokens, int heads, int rank,
+                               int rot_dim, int64_t qrot_token_stride, int64_t qrot_head_stride, float scale,
+                               SP_SEQ_PARAMS, int dtype, void* stream);
+
+/* Router: z = router x in fp32, s = sigmoid(z), choice = s + correction; with groups > 1 only experts of the `keep`
+ * groups with the largest (sum of the group's two largest choices) can win; ids [T, top] = the largest choices,
+ * weights [T, top] = their s.                                                                                     */
+SP_API int sp_moe_route(int32_t* ids, float* weights, const void* x, int64_t x_stride, const float* router,
+                        const float* correction, int64_t num_tokens, int width, int experts, int top, int groups,
+                        int keep, int dtype, void* stream);
+/* (token, expert) pairs ordered by expert: offsets [experts + 1], order[pos] = pair, place[pair] = pos */
+SP_API int sp_moe_align(int32_t* offsets, int32_t* order, int32_t* place, const int32_t* ids, int pairs, int experts,
+                        void* stream);
+/* out[pos, :] = w[expert(pos)] a[row(pos)], w [experts, n, k]; row(pos) = order[pos] / row_div, or pos when order is null */
+SP_API int sp_moe_grouped_gemm(void* out, const void* a, const void* w, const int32_t* offsets, const int32_t* order,
+                               int row_div, int pairs, int n, int k, int experts, int64_t a_stride, int64_t out_stride,
+                               int dtype, void* stream);
+/* out[p, f] = g * sigmoid(alpha g) * (u + 1), g = min(gu[p, f], limit), u = clamp(gu[p, ff + f], -limit, limit) */
+SP_API int sp_moe_glu(void* out, const void* gu, int64_t pairs, int ff, float limit, float alpha, int dtype, void* stream);
+/* out[t] = sum over k < top, in that order, of weights[t, k] * z[place[t * top + k]] */
+SP_API int sp_moe_combine(void* out, const void* z, const int32_t* place, const float* weights, int64_t num_tokens,
+                          int width, int top, int64_t out_stride, int dtype, void* stream);
 
 #ifdef __cplusplus
 }

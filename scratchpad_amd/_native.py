@@ -50,6 +50,7 @@ def _kv_dt(buf: torch.Tensor, q: torch.Tensor, what: str) -> int:
 _vp, _i64, _i32, _f32, _sz = (ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_float,
                               ctypes.c_size_t)
 
+_SEQ = [_vp, _vp, _vp, _vp, _vp, _vp, _i32, _i32]
 # name -> (restype, argtypes); must list every symbol include/scratchpad_hip.h declares
 SIGNATURES = {
     "sp_abi_version": (_i32, []),
@@ -101,7 +102,36 @@ SIGNATURES = {
     "sp_fused_allreduce_add_rmsnorm": (_i32, [_vp, _vp, _vp, _i64, _i32, _i64, _i64, _f32, _i32, _vp, _i32, _i32,
                                               _sz, _i64, _vp, _vp]),
     "sp_gemm_skinny": (_i32, [_vp, _vp, _vp, _i32, _i32, _i32, _i64, _i64, _i64, _i32, _i32, _vp]),
+    # ---- ABI 10 (_SEQ: the header's SP_SEQ_PARAMS)
+    "sp_bigram_rows": (_i32, [_vp, _vp, _vp, _i64, *_SEQ, _i64, _i64, _i64, _vp]),
+    "sp_save_last_token": (_i32, [_vp, _vp, *_SEQ, _vp]),
+    "sp_save_last_rows": (_i32, [_vp, _i64, _vp, _i64, _i32, *_SEQ, _vp]),
+    "sp_embed_bigram_norm": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i32, _i64, _i64, _f32, _i32, _vp]),
+    "sp_add_scalar_norm": (_i32, [_vp, _vp, _vp, _vp, _i64, _i32, _i64, _i64, _i64, _f32, _i32, _vp]),
+    "sp_scalar_norm": (_i32, [_vp, _vp, _vp, _i64, _i32, _i64, _i64, _f32, _i32, _vp]),
+    "sp_polynorm": (_i32, [_vp, _vp, _vp, _i64, _i32, _i64, _i64, _f32, _i32, _vp]),
+    "sp_gate_heads": (_i32, [_vp, _vp, _vp, _i64, _i32, _i32, _i64, _i32, _vp]),
+    "sp_token_shift": (_i32, [_vp, _vp, _vp, _vp, _i64, _i64, _i32, _i32, _i64, *_SEQ, _i32, _vp]),
+    "sp_wkv_decay": (_i32, [_vp, _vp, _vp, _vp, _i64, _i32, _i32, _i64, _i32, _vp]),
+    "sp_wkv_recurrence": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i32, _i32, _i64, _i64, _i64, _i64,
+                                 _i64, _f32, *_SEQ, _i32, _vp]),
+    "sp_rotary_interleaved": (_i32, [_vp, _vp, _vp, _f32, _i64, _i32, _i32, _i64, _i64, _i32, _i32, _vp]),
+    "sp_latent_kv_store": (_i32, [_vp, _i64, _vp, _i64, _vp, _vp, _vp, _f32, _vp, _i64, _i32, _i32, _i32, _f32, _i32, _vp]),
+    "sp_latent_attention": (_i32, [_vp, _vp, _vp, _vp, _i64, _vp, _i64, _i64, _i32, _i32, _i32, _i64, _i64, _f32, *_SEQ,
+                                   _i32, _vp]),
+    "sp_moe_route": (_i32, [_vp, _vp, _vp, _i64, _vp, _vp, _i64, _i32, _i32, _i32, _i32, _i32, _i32, _vp]),
+    "sp_moe_align": (_i32, [_vp, _vp, _vp, _vp, _i32, _i32, _vp]),
+    "sp_moe_grouped_gemm": (_i32, [_vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _i64, _i64, _i32, _vp]),
+    "sp_moe_glu": (_i32, [_vp, _vp, _i64, _i32, _f32, _f32, _i32, _vp]),
+    "sp_moe_combine": (_i32, [_vp, _vp, _vp, _vp, _i64, _i32, _i32, _i64, _i32, _vp]),
 }
+
+
+def _not_built(name: str):
+    def missing(*_a, **_k):
+        raise RuntimeError(f"{name} is not in this build of {_LIB_PATH} (it was made of the sources of one model family): "
+                           "run `python -m scratchpad_amd.build` for the whole library")
+    return missing
 
 
 def lib_path() -> str:
@@ -119,10 +149,15 @@ def load() -> ctypes.CDLL:
             "(or __graft_entry__.build()); there is no fallback path")
     lib = ctypes.CDLL(_LIB_PATH)
     for name, (res, args) in SIGNATURES.items():
-        fn = getattr(lib, name)
+        try:
+            fn = getattr(lib, name)
+        except AttributeError:
+            # a library built from the sources of one model family (build.build_native(only=...)): the rest raises on use
+            setattr(lib, name, _not_built(name))
+            continue
         fn.restype = res
         fn.argtypes = args
-    if lib.sp_abi_version() != 9:
+    if lib.sp_abi_version() != 10:
         raise RuntimeError("libscratchpad_hip.so ABI version mismatch")
     _lib = lib
     return lib
@@ -872,3 +907,268 @@ def linear(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
 
 def _feeds_a_measured_shape(width: int) -> bool:
     return any(k == width for (_n, k) in _LIBRARY_ROWS)
+
+
+# --------------------------------------------------------------------------- per-sequence state, latent attention, experts
+class SeqParams:
+    """The header's SP_SEQ_PARAMS of one step, built once per forward (``from_forward_batch``) and handed to every kernel
+    that reads or writes per-request state.  Holds the tensors, so the pointers stay valid while it lives."""
+
+    def __init__(self, req_pool_indices: torch.Tensor, seq_lens: torch.Tensor, extend_seq_lens=None,
+                 extend_prefix_lens=None, extend_start_loc=None, token_req=None):
+        _gpu(req_pool_indices, seq_lens, extend_seq_lens, extend_prefix_lens, extend_start_loc, token_req)
+        if req_pool_indices.dtype not in (torch.int32, torch.int64):
+            raise RuntimeError("req_pool_indices must be int32 or int64")
+        if seq_lens.dtype != req_pool_indices.dtype:
+            seq_lens = seq_lens.to(req_pool_indices.dtype)
+        self.req_pool_indices, self.seq_lens = req_pool_indices.contiguous(), seq_lens.contiguous()
+        ext = (extend_seq_lens, extend_prefix_lens, extend_start_loc, token_req)
+        if any(t is not None for t in ext):
+            if any(t is None or t.dtype != torch.int32 for t in ext):
+                raise RuntimeError("a multi-token step needs extend_seq_lens, extend_prefix_lens, extend_start_loc and "
+                                   "token_req, all int32")
+            ext = tuple(t.contiguous() for t in ext)
+        self.extend_seq_lens, self.extend_prefix_lens, self.extend_start_loc, self.token_req = ext
+        self.batch_size = int(self.req_pool_indices.shape[0])
+        self.num_tokens = self.batch_size if token_req is None else int(self.token_req.shape[0])
+        self.args = [self.req_pool_indices.data_ptr(), self.seq_lens.data_ptr(), _ptr(self.extend_seq_lens),
+                     _ptr(self.extend_prefix_lens), _ptr(self.extend_start_loc), _ptr(self.token_req),
+                     int(self.req_pool_indices.dtype == torch.int64), self.batch_size]
+
+    @classmethod
+    def from_forward_batch(cls, fb) -> "SeqParams":
+        if fb.forward_mode.is_decode():
+            return cls(fb.req_pool_indices, fb.seq_lens)
+        bs = fb.batch_size
+        token_req = torch.repeat_interleave(torch.arange(bs, dtype=torch.int32, device=fb.extend_seq_lens.device),
+                                            fb.extend_seq_lens.long(), output_size=fb.extend_num_tokens)
+        return cls(fb.req_pool_indices, fb.seq_lens, fb.extend_seq_lens, fb.extend_prefix_lens, fb.extend_start_loc,
+                   token_req)
+
+
+def _f32(t: torch.Tensor, what: str) -> torch.Tensor:
+    if t.dtype != torch.float32 or not t.is_cuda or not t.is_contiguous():
+        raise RuntimeError(f"{what} must be a contiguous fp32 device tensor")
+    return t
+
+
+def _mat(t: torch.Tensor, what: str) -> torch.Tensor:
+    if t.dim() != 2 or t.stride(1) != 1:
+        raise RuntimeError(f"{what} must be [rows, n] with a contiguous last dimension, got {tuple(t.shape)} {tuple(t.stride())}")
+    return t
+
+
+def bigram_rows(ids: torch.Tensor, last_token: torch.Tensor, seq: SeqParams, buckets: int, mul_prev: int,
+                mul_cur: int) -> torch.Tensor:
+    _gpu(ids, last_token)
+    if ids.dtype != torch.int64 or last_token.dtype != torch.int64 or ids.shape[0] != seq.num_tokens:
+        raise RuntimeError("bigram_rows: ids [num_tokens] and last_token must be int64")
+    rows = torch.empty(ids.shape[0], dtype=torch.int32, device=ids.device)
+    _check(load().sp_bigram_rows(rows.data_ptr(), ids.data_ptr(), last_token.data_ptr(), ids.shape[0], *seq.args,
+                                 buckets, mul_prev, mul_cur, _stream()), "sp_bigram_rows")
+    return rows
+
+
+def save_last_token(last_token: torch.Tensor, ids: torch.Tensor, seq: SeqParams) -> None:
+    _check(load().sp_save_last_token(last_token.data_ptr(), ids.data_ptr(), *seq.args, _stream()), "sp_save_last_token")
+
+
+def save_last_rows(state: torch.Tensor, x: torch.Tensor, seq: SeqParams) -> None:
+    _f32(state, "state")
+    _mat(x, "x")
+    if x.dtype != torch.float32 or state.shape[-1] != x.shape[1] or x.shape[0] != seq.num_tokens:
+        raise RuntimeError("save_last_rows: x [num_tokens, width] fp32, state [slots, width]")
+    _check(load().sp_save_last_rows(state.data_ptr(), state.stride(0), x.data_ptr(), x.stride(0), x.shape[1], *seq.args,
+                                    _stream()), "sp_save_last_rows")
+
+
+def embed_bigram_norm(embed: torch.Tensor, bigram: torch.Tensor, ids: torch.Tensor, rows: torch.Tensor,
+                      gain: torch.Tensor, eps: float):
+    """(x fp32 [T, W], the same in the tables' dtype)"""
+    _gpu(embed, bigram, ids, rows)
+    _f32(gain, "gain")
+    if embed.dtype != bigram.dtype or embed.shape[1] != bigram.shape[1] or not embed.is_contiguous() or not bigram.is_contiguous():
+        raise RuntimeError("embed_bigram_norm: tables must share dtype and width and be contiguous")
+    T, W = ids.shape[0], embed.shape[1]
+    x = torch.empty((T, W), dtype=torch.float32, device=embed.device)
+    lo = x if embed.dtype == torch.float32 else empty_rows(T, W, embed.dtype, embed.device)
+    _check(load().sp_embed_bigram_norm(x.data_ptr(), None if lo is x else lo.data_ptr(), embed.data_ptr(), bigram.data_ptr(),
+                                       ids.data_ptr(), rows.data_ptr(), gain.data_ptr(), T, W, x.stride(0), lo.stride(0),
+                                       eps, _dt(embed), _stream()), "sp_embed_bigram_norm")
+    return x, lo
+
+
+def add_scalar_norm(x: torch.Tensor, y: torch.Tensor, gain: torch.Tensor, eps: float, want_lo: bool = True):
+    """x += y / rms(y) * gain in place (x fp32); returns x in y's dtype for the next projection (x itself when fp32)"""
+    _mat(x, "x"), _mat(y, "y"), _f32(gain, "gain")
+    if x.dtype != torch.float32 or x.shape != y.shape:
+        raise RuntimeError("add_scalar_norm: x fp32 [T, W], y [T, W]")
+    lo = None
+    if want_lo and y.dtype != torch.float32:
+        lo = empty_rows(x.shape[0], x.shape[1], y.dtype, x.device)
+    _check(load().sp_add_scalar_norm(x.data_ptr(), _ptr(lo), y.data_ptr(), gain.data_ptr(), x.shape[0], x.shape[1],
+                                     x.stride(0), 0 if lo is None else lo.stride(0), y.stride(0), eps, _dt(y), _stream()),
+           "sp_add_scalar_norm")
+    return x if lo is None else lo
+
+
+def scalar_norm(x: torch.Tensor, gain: torch.Tensor, eps: float, dtype: torch.dtype) -> torch.Tensor:
+    _mat(x, "x"), _f32(gain, "gain")
+    if x.dtype != torch.float32:
+        raise RuntimeError("scalar_norm: x must be fp32")
+    out = empty_rows(x.shape[0], x.shape[1], dtype, x.device)
+    _check(load().sp_scalar_norm(out.data_ptr(), x.data_ptr(), gain.data_ptr(), x.shape[0], x.shape[1], x.stride(0),
+                                 out.stride(0), eps, _DTYPES[dtype], _stream()), "sp_scalar_norm")
+    return out
+
+
+def polynorm(z: torch.Tensor, coef: torch.Tensor, eps: float) -> torch.Tensor:
+    _mat(z, "z"), _f32(coef, "coef")
+    out = empty_rows(z.shape[0], z.shape[1], z.dtype, z.device)
+    _check(load().sp_polynorm(out.data_ptr(), z.data_ptr(), coef.data_ptr(), z.shape[0], z.shape[1], z.stride(0),
+                              out.stride(0), eps, _dt(z), _stream()), "sp_polynorm")
+    return out
+
+
+def gate_heads(o: torch.Tensor, g: torch.Tensor) -> torch.Tensor:
+    """o [H, T, D] contiguous, g [T, H] -> [T, H * D] = o * sigmoid(g) per head"""
+    _mat(g, "g")
+    if o.dim() != 3 or not o.is_contiguous() or g.shape != (o.shape[1], o.shape[0]) or g.dtype != o.dtype:
+        raise RuntimeError("gate_heads: o [H, T, D] contiguous, g [T, H] of the same dtype")
+    H, T, D = o.shape
+    out = empty_rows(T, H * D, o.dtype, o.device)
+    _check(load().sp_gate_heads(out.data_ptr(), o.data_ptr(), g.data_ptr(), T, H, D, g.stride(0), _dt(o), _stream()),
+           "sp_gate_heads")
+    return out
+
+
+def token_shift(x: torch.Tensor, mu: torch.Tensor, shift_state: torch.Tensor, seq: SeqParams, dtype: torch.dtype) -> torch.Tensor:
+    """[mixes, T, W] in dtype: x[t] + (x[t-1] - x[t]) * mu[m]"""
+    _mat(x, "x"), _f32(mu, "mu"), _f32(shift_state, "shift_state")
+    if x.dtype != torch.float32 or mu.shape[1] != x.shape[1] or shift_state.shape[1] != x.shape[1] or x.shape[0] != seq.num_tokens:
+        raise RuntimeError("token_shift: x fp32 [num_tokens, W], mu [mixes, W], shift_state [slots, W]")
+    out = torch.empty((mu.shape[0] * x.shape[0] + ROW_SLACK, x.shape[1]), dtype=dtype, device=x.device)
+    _check(load().sp_token_shift(out.data_ptr(), x.data_ptr(), mu.data_ptr(), shift_state.data_ptr(), shift_state.stride(0),
+                                 x.shape[0], x.shape[1], mu.shape[0], x.stride(0), *seq.args, _DTYPES[dtype], _stream()),
+           "sp_token_shift")
+    return out[:mu.shape[0] * x.shape[0]].view(mu.shape[0], x.shape[0], x.shape[1])
+
+
+def wkv_decay(a: torch.Tensor, w2t: torch.Tensor, w0: torch.Tensor) -> torch.Tensor:
+    _mat(a, "a"), _f32(w2t, "w2t"), _f32(w0, "w0")
+    if w2t.shape[0] != a.shape[1] or w0.shape[0] != w2t.shape[1]:
+        raise RuntimeError("wkv_decay: a [T, rank], w2t [rank, channels], w0 [channels]")
+    out = torch.empty((a.shape[0], w2t.shape[1]), dtype=torch.float32, device=a.device)
+    _check(load().sp_wkv_decay(out.data_ptr(), a.data_ptr(), w2t.data_ptr(), w0.data_ptr(), a.shape[0], w2t.shape[1],
+                               w2t.shape[0], a.stride(0), _dt(a), _stream()), "sp_wkv_decay")
+    return out
+
+
+def wkv_recurrence(r, k, v, g, decay, u, norm_w, state, seq: SeqParams, heads: int, dim: int, eps: float) -> torch.Tensor:
+    for name, t in (("r", r), ("k", k), ("v", v), ("g", g)):
+        _mat(t, name)
+        if t.dtype != r.dtype or t.shape != (seq.num_tokens, heads * dim):
+            raise RuntimeError(f"wkv_recurrence: {name} must be [num_tokens, heads * dim] of one dtype")
+    _f32(decay, "decay"), _f32(u, "u"), _f32(norm_w, "norm_w"), _f32(state, "state")
+    if decay.shape != r.shape or u.numel() != heads * dim or norm_w.numel() != heads * dim or \
+            state.shape[1:] != (heads, dim, dim):
+        raise RuntimeError("wkv_recurrence: decay [T, H*D], u [H, D], norm_w [H*D], state [slots, H, D, D]")
+    out = empty_rows(r.shape[0], heads * dim, r.dtype, r.device)
+    _check(load().sp_wkv_recurrence(out.data_ptr(), r.data_ptr(), k.data_ptr(), v.data_ptr(), g.data_ptr(), decay.data_ptr(),
+                                    u.data_ptr(), norm_w.data_ptr(), state.data_ptr(), state.stride(0), heads, dim,
+                                    r.stride(0), k.stride(0), v.stride(0), g.stride(0), out.stride(0), eps, *seq.args,
+                                    _dt(r), _stream()), "sp_wkv_recurrence")
+    return out
+
+
+def rotary_interleaved(x: torch.Tensor, positions: torch.Tensor, freq: torch.Tensor, mag: float, offset: int = 0) -> None:
+    """in place on x [T, H, n]: the pairs of x[..., offset : offset + 2 * len(freq)]"""
+    _f32(freq, "freq")
+    if x.dim() != 3 or x.stride(2) != 1 or positions.dtype != torch.int64 or offset + 2 * freq.shape[0] > x.shape[2]:
+        raise RuntimeError("rotary_interleaved: x [T, H, n] with contiguous last dimension, int64 positions")
+    _check(load().sp_rotary_interleaved(x.data_ptr(), positions.data_ptr(), freq.data_ptr(), mag, x.shape[0], x.shape[1],
+                                        2 * freq.shape[0], x.stride(0), x.stride(1), offset, _dt(x), _stream()),
+           "sp_rotary_interleaved")
+
+
+def latent_kv_store(pool: torch.Tensor, dkv: torch.Tensor, norm_w: torch.Tensor, positions: torch.Tensor,
+                    freq: torch.Tensor, mag: float, loc: torch.Tensor, rank: int, eps: float) -> None:
+    _mat(pool, "pool"), _mat(dkv, "dkv"), _f32(norm_w, "norm_w"), _f32(freq, "freq")
+    rot_dim = dkv.shape[1] - rank
+    if pool.dtype != dkv.dtype or pool.shape[1] != dkv.shape[1] or norm_w.shape[0] != rank or rot_dim < 2 * freq.shape[0] \
+            or loc.dtype != torch.int64 or positions.dtype != torch.int64 or loc.shape[0] != dkv.shape[0]:
+        raise RuntimeError("latent_kv_store: pool [P, rank + rot], dkv [T, rank + rot] of one dtype, int64 loc / positions")
+    _check(load().sp_latent_kv_store(pool.data_ptr(), pool.stride(0), dkv.data_ptr(), dkv.stride(0), norm_w.data_ptr(),
+                                     positions.data_ptr(), freq.data_ptr(), mag, loc.data_ptr(), dkv.shape[0], rank, rot_dim,
+                                     2 * freq.shape[0], eps, _dt(dkv), _stream()), "sp_latent_kv_store")
+
+
+def latent_attention(q_lat: torch.Tensor, q_rot: torch.Tensor, pool: torch.Tensor, req_to_token: torch.Tensor,
+                     seq: SeqParams, scale: float) -> torch.Tensor:
+    """q_lat [H, T, rank] contiguous; q_rot [T, H, rot] (a view: strides are taken); pool [P, rank + rot]; -> [H, T, rank]"""
+    _mat(pool, "pool")
+    H, T, rank = q_lat.shape
+    if not q_lat.is_contiguous() or q_rot.dim() != 3 or q_rot.stride(2) != 1 or q_rot.shape[:2] != (T, H) or \
+            pool.shape[1] != rank + q_rot.shape[2] or q_lat.dtype != pool.dtype or q_rot.dtype != pool.dtype or \
+            req_to_token.dtype != torch.int32 or T != seq.num_tokens:
+        raise RuntimeError("latent_attention: shapes / dtypes do not fit")
+    out = torch.empty((H, T, rank), dtype=q_lat.dtype, device=q_lat.device)
+    _check(load().sp_latent_attention(out.data_ptr(), q_lat.data_ptr(), q_rot.data_ptr(), pool.data_ptr(), pool.stride(0),
+                                      req_to_token.data_ptr(), req_to_token.stride(0), T, H, rank, q_rot.shape[2],
+                                      q_rot.stride(0), q_rot.stride(1), scale, *seq.args, _dt(q_lat), _stream()),
+           "sp_latent_attention")
+    return out
+
+
+def moe_route(x: torch.Tensor, router: torch.Tensor, correction: torch.Tensor, top: int, groups: int, keep: int):
+    """(ids int32 [T, top], weights fp32 [T, top])"""
+    _mat(x, "x"), _f32(router, "router"), _f32(correction, "correction")
+    T, E = x.shape[0], router.shape[0]
+    ids = torch.empty((T, top), dtype=torch.int32, device=x.device)
+    weights = torch.empty((T, top), dtype=torch.float32, device=x.device)
+    _check(load().sp_moe_route(ids.data_ptr(), weights.data_ptr(), x.data_ptr(), x.stride(0), router.data_ptr(),
+                               correction.data_ptr(), T, x.shape[1], E, top, groups, keep, _dt(x), _stream()), "sp_moe_route")
+    return ids, weights
+
+
+def moe_align(ids: torch.Tensor, experts: int):
+    """(offsets [E + 1], order [P], place [P]) int32: the (token, expert) pairs ordered by expert"""
+    P = ids.numel()
+    offsets = torch.empty(experts + 1, dtype=torch.int32, device=ids.device)
+    order = torch.empty(P, dtype=torch.int32, device=ids.device)
+    place = torch.empty(P, dtype=torch.int32, device=ids.device)
+    _check(load().sp_moe_align(offsets.data_ptr(), order.data_ptr(), place.data_ptr(), ids.data_ptr(), P, experts, _stream()),
+           "sp_moe_align")
+    return offsets, order, place
+
+
+def moe_grouped_gemm(a: torch.Tensor, w: torch.Tensor, offsets: torch.Tensor, pairs: int, order: Optional[torch.Tensor] = None,
+                     row_div: int = 1) -> torch.Tensor:
+    """out [pairs, N]: row pos = w[expert of pos] @ a[order[pos] // row_div] (a[pos] without order); w [E, N, K]"""
+    _mat(a, "a")
+    if w.dim() != 3 or not w.is_contiguous() or w.dtype != a.dtype or w.shape[2] != a.shape[1]:
+        raise RuntimeError("moe_grouped_gemm: w [E, N, K] contiguous of a's dtype")
+    E, N, K = w.shape
+    out = torch.empty((pairs, N), dtype=a.dtype, device=a.device)
+    _check(load().sp_moe_grouped_gemm(out.data_ptr(), a.data_ptr(), w.data_ptr(), offsets.data_ptr(), _ptr(order), row_div,
+                                      pairs, N, K, E, a.stride(0), out.stride(0), _dt(a), _stream()), "sp_moe_grouped_gemm")
+    return out
+
+
+def moe_glu(gu: torch.Tensor, limit: float, alpha: float) -> torch.Tensor:
+    if gu.dim() != 2 or not gu.is_contiguous() or gu.shape[1] % 2:
+        raise RuntimeError("moe_glu: gu [P, 2 * ff] contiguous")
+    out = torch.empty((gu.shape[0], gu.shape[1] // 2), dtype=gu.dtype, device=gu.device)
+    _check(load().sp_moe_glu(out.data_ptr(), gu.data_ptr(), gu.shape[0], gu.shape[1] // 2, limit, alpha, _dt(gu), _stream()),
+           "sp_moe_glu")
+    return out
+
+
+def moe_combine(z: torch.Tensor, place: torch.Tensor, weights: torch.Tensor) -> torch.Tensor:
+    T, top = weights.shape
+    if z.dim() != 2 or not z.is_contiguous() or z.shape[0] != T * top:
+        raise RuntimeError("moe_combine: z [T * top, W] contiguous")
+    out = empty_rows(T, z.shape[1], z.dtype, z.device)
+    _check(load().sp_moe_combine(out.data_ptr(), z.data_ptr(), place.data_ptr(), weights.data_ptr(), T, z.shape[1], top,
+                                 out.stride(0), _dt(z), _stream()), "sp_moe_combine")
+    return out

@@ -29,6 +29,13 @@ PER_FILE_FLAGS = {"elementwise.hip": ["-ffp-contract=off"], "allreduce.hip": ["-
                   # accumulation registers belong to its assembly text alone: compile_w64 below / tools/w64_asm.py.  The
                   # atomic optimizer would turn the persistent form's ticket draw into atomic + full wait + broadcast.
                   "extend_w64.hip": ["-fno-honor-nans", "-fno-slp-vectorize", "-std=c++20", "-mllvm", "-amdgpu-atomic-optimizer-strategy=None"]}
+# fp32 state and residual kernels: scalar fp32 instructions only (no packed-fp32 forms)
+_NO_PACKED_F32 = ["-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unknown-warning-option"]
+for _f in ("scalar_norm.hip", "wkv.hip", "latent_attention.hip", "moe.hip"):
+    PER_FILE_FLAGS[_f] = list(_NO_PACKED_F32)
+# Sources a model family needs beyond these: a model class names them (NATIVE_SOURCES) and build_native(only=...) makes
+# a library of just those, so the first start of a small model does not compile the attention kernels of another.
+CORE_SOURCES = ["elementwise.hip", "gemm_skinny.hip", "sampling.hip"]
 
 
 def _newer(target, deps):
@@ -110,8 +117,26 @@ def compile_w64(src: str, obj: str, extra=(), verbose: bool = True) -> str:
     return obj
 
 
-def build_native(force: bool = False, verbose: bool = True) -> str:
+def built_sources(lib: str = LIB):
+    """basenames of the sources the library on disk was made of (None: no library, or one without a stamp)"""
+    stamp = lib + ".sources"
+    if not (os.path.exists(lib) and os.path.exists(stamp)):
+        return None
+    return [l for l in open(stamp).read().splitlines() if l.endswith(".hip")]
+
+
+def build_native(force: bool = False, verbose: bool = True, only=None) -> str:
+    """The whole library, or (``only``: source basenames) a library of CORE_SOURCES plus those.  A library that already
+    holds what is asked for, and is newer than its sources, is kept; a partial one is replaced by a full build."""
     srcs = sorted(glob.glob(os.path.join(CSRC, "*.hip")))
+    if only is not None:
+        want = set(CORE_SOURCES) | set(only)
+        have = built_sources()
+        if not force and have is not None and want <= set(have):
+            srcs = [x for x in srcs if os.path.basename(x) in have]      # up to date? checked below against ITS sources
+        else:
+            srcs = [x for x in srcs if os.path.basename(x) in want]
+    partial = not any(os.path.basename(x) == "extend_w64.hip" for x in srcs)
     hdrs = sorted(glob.glob(os.path.join(CSRC, "*.h"))) + sorted(glob.glob(os.path.join(CSRC, "*.inc"))) + [
         os.path.join(ROOT, "include", "scratchpad_hip.h"), os.path.join(ROOT, "tools", "w64_asm.py")]
     # (the library also has to be made of exactly these sources and flags: a source removed - or a flag changed - leaves
@@ -122,7 +147,8 @@ def build_native(force: bool = False, verbose: bool = True) -> str:
                         ["compiler: " + _hipcc_version()])
     same = os.path.exists(stamp) and open(stamp).read() == made_of
     if not force and same and _newer(LIB, srcs + hdrs):
-        check_w64_descriptors(LIB)       # (cheap: reads the ELF; a library somebody linked by hand fails here)
+        if not partial:
+            check_w64_descriptors(LIB)   # (cheap: reads the ELF; a library somebody linked by hand fails here)
         return LIB
     force = force or not same
     os.makedirs(OBJ, exist_ok=True)
@@ -146,7 +172,8 @@ def build_native(force: bool = False, verbose: bool = True) -> str:
     if verbose:
         print(" ".join(cmd), flush=True)
     subprocess.run(cmd, check=True)
-    check_w64_descriptors(LIB, verbose)
+    if not partial:
+        check_w64_descriptors(LIB, verbose)
     with open(stamp, "w") as f:
         f.write(made_of)
     return LIB
