@@ -513,3 +513,68 @@ class HipAttnBackend(AttentionBackend):
             layer.scaling, layer.logit_cap, max_len, chunk, ws, kv_start, plan,
             k_scale=k_scale, v_scale=v_scale, max_slots=slots, ranges=ranges)
         return o
+
+
+# --------------------------------------------------------------------------- latent (compressed key/value) attention
+class LatentAttention(nn.Module):
+    """Layer-local constants of an attention layer over a LatentTokenToKVPool (the counterpart of RadixAttention): the
+    pool row of a token is [normed latent (rank) | rotated shared key part (rot_dim)]; every head's key and value are
+    products of the latent, folded into the query and the output by the model (q_lat = W_uk^T q, out = W_uv o_lat)."""
+
+    def __init__(self, num_heads: int, rank: int, rot_dim: int, scaling: float, layer_id: int):
+        super().__init__()
+        self.tp_q_head_num = num_heads
+        self.rank, self.rot_dim = rank, rot_dim
+        self.scaling = scaling
+        self.layer_id = layer_id
+
+    def forward(self, q_lat, q_rot, forward_batch: "ForwardBatch"):
+        """q_lat [H, T, rank], q_rot [T, H, rot_dim] (rotated) -> o_lat [H, T, rank]; the step's rows are in the pool"""
+        return forward_batch.attn_backend.forward_latent(q_lat, q_rot, self, forward_batch)
+
+
+class SequenceBackend(AttentionBackend):
+    """Backend of models whose layers read per-request state through the step's request table instead of a planned
+    key/value gather: latent attention layers (LatentTokenToKVPool) and recurrent layers (RecurrentStatePool).  Its
+    per-step metadata is the kernels' request description (_native.SeqParams), built once per forward; launches read
+    req_pool_indices / seq_lens from the batch's own tensors, so a captured decode step replays on the graph runner's
+    static buffers with nothing to rebuild."""
+
+    def __init__(self, model_runner):
+        super().__init__()
+        _native.load()
+        self.device = model_runner.device
+        self.max_context_len = model_runner.model_config.context_len
+        self.forward_metadata = None
+
+    def init_forward_metadata(self, forward_batch: "ForwardBatch"):
+        self.forward_metadata = _native.SeqParams.from_forward_batch(forward_batch)
+
+    @property
+    def seq(self) -> "_native.SeqParams":
+        return self.forward_metadata
+
+    def init_cuda_graph_state(self, max_bs: int):
+        pass
+
+    def init_forward_metadata_capture_cuda_graph(self, bs, num_tokens, req_pool_indices, seq_lens, encoder_lens,
+                                                 forward_mode, spec_info=None):
+        assert forward_mode.is_decode(), "only decode is captured"
+        self.forward_metadata = _native.SeqParams(req_pool_indices[:bs], seq_lens[:bs])
+
+    def init_forward_metadata_replay_cuda_graph(self, bs, req_pool_indices, seq_lens, seq_lens_sum, encoder_lens,
+                                                forward_mode, spec_info=None, seq_lens_cpu=None):
+        pass                      # the captured launches read the static buffers
+
+    def get_cuda_graph_seq_len_fill_value(self):
+        return 1                  # a padded row is a sequence's first token on the reserved request row / dummy slot
+
+    def forward_latent(self, q_lat, q_rot, layer: LatentAttention, forward_batch: "ForwardBatch"):
+        pool = forward_batch.token_to_kv_pool.get_key_buffer(layer.layer_id)
+        return _native.latent_attention(q_lat, q_rot, pool, forward_batch.req_to_token_pool.req_to_token, self.seq,
+                                        layer.scaling)
+
+    def forward_decode(self, q, k, v, layer, forward_batch, save_kv_cache: bool = True):
+        raise NotImplementedError("this backend serves latent attention layers (forward_latent)")
+
+    forward_extend = forward_decode

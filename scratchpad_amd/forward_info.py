@@ -106,6 +106,8 @@ class ModelWorkerBatch:
     # stand-in for the (un-hosted) vision tower: projected + flattened vision states of the requests
     # whose encoder is not cached, [sum(encoder_lens_need), hidden] (mllama.py:966-979)
     encoder_states: Optional[torch.Tensor] = None
+    # int64 indices into the step's token rows: return the logits of exactly these rows (prompt scoring, trace replay)
+    logit_rows: Optional[torch.Tensor] = None
 
 
 @dataclass
@@ -164,6 +166,9 @@ class ForwardBatch:
     mrope_positions: torch.Tensor = None
     # ---- not in the reference (kept behind its fields)
     encoder_states: Optional[torch.Tensor] = None    # see ModelWorkerBatch
+    state_pool: Any = None                           # pool.RecurrentStatePool of models with per-request state
+    # rows of the step (indices into its token rows) whose logits are returned instead of each request's last one
+    logit_rows: Optional[torch.Tensor] = None
 
     @classmethod
     def init_new(cls, batch: ModelWorkerBatch, model_runner) -> "ForwardBatch":
@@ -189,7 +194,8 @@ class ForwardBatch:
             token_to_kv_pool=model_runner.token_to_kv_pool, attn_backend=model_runner.attn_backend,
             spec_algorithm=batch.spec_algorithm, spec_info=batch.spec_info,
             capture_hidden_mode=batch.capture_hidden_mode, input_embeds=batch.input_embeds,
-            encoder_states=batch.encoder_states,
+            encoder_states=batch.encoder_states, state_pool=getattr(model_runner, "state_pool", None),
+            logit_rows=(None if batch.logit_rows is None else batch.logit_rows.to(device, non_blocking=True)),
             extend_input_logprob_token_ids_gpu=(None if batch.extend_input_logprob_token_ids is None else
                                                 batch.extend_input_logprob_token_ids.to(device, non_blocking=True)))
         if batch.global_num_tokens is not None:

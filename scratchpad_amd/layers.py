@@ -218,3 +218,70 @@ def get_rope(head_size: int, rotary_dim: int, max_position: int, base: int,
         raise ValueError(f"Unknown RoPE scaling type {scaling_type}")
     _ROPE_DICT[key] = rope
     return rope
+
+
+# --------------------------------------------------------------------------- fp32-stream norms, PolyNorm, table-free rotary
+class ScalarRMSNorm(nn.Module):
+    """RMS norm with ONE gain for all coordinates, applied to a sublayer's OUTPUT before it joins an fp32 residual
+    stream: ``add_into(x, y)`` is x += y / rms(y) * g in place and returns the new x in y's dtype (what the next
+    projection reads); ``forward(x, dtype)`` is the plain norm of the stream (a model's final norm)."""
+
+    def __init__(self, eps: float = 1e-6) -> None:
+        super().__init__()
+        self.weight = nn.Parameter(torch.ones(1, dtype=torch.float32), requires_grad=False)
+        self.variance_epsilon = eps
+
+    def add_into(self, x: torch.Tensor, y: torch.Tensor, want_lo: bool = True) -> torch.Tensor:
+        return _native.add_scalar_norm(x, y, self.weight.data, self.variance_epsilon, want_lo)
+
+    def forward(self, x: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
+        return _native.scalar_norm(x, self.weight.data, self.variance_epsilon, dtype)
+
+
+class PolyNorm(nn.Module):
+    """a N(z) + b N(z^2) + c N(z^3) + e with N = division by the root mean square over the row; weight = (a, b, c, e)"""
+
+    def __init__(self, eps: float = 1e-6) -> None:
+        super().__init__()
+        self.weight = nn.Parameter(torch.tensor([1.0, 0.0, 0.0, 0.0], dtype=torch.float32), requires_grad=False)
+        self.variance_epsilon = eps
+
+    def forward(self, z: torch.Tensor) -> torch.Tensor:
+        return _native.polynorm(z, self.weight.data, self.variance_epsilon)
+
+
+def yarn_blend(dims: int, base: float, factor: float, original: float, fast: float, slow: float) -> torch.Tensor:
+    """Rotary frequencies f_i = base^(-2i/dims), i < dims/2, blended with f_i / factor along a linear ramp between the
+    (fractional) dimensions that complete `fast` and `slow` turns inside `original` positions: below the ramp the
+    frequency stays, above it is divided by the factor.  float64."""
+    f = torch.tensor([base ** (-2.0 * i / dims) for i in range(dims // 2)], dtype=torch.float64)
+
+    def dim_of(turns: float) -> float:
+        return dims * math.log(original / (2 * math.pi * turns)) / (2 * math.log(base))
+    lo = max(math.floor(dim_of(fast)), 0)
+    hi = min(math.ceil(dim_of(slow)), dims - 1)
+    ramp = torch.clamp((torch.arange(dims // 2, dtype=torch.float64) - lo) / max(hi - lo, 0.001), 0, 1)
+    return f / factor * ramp + f * (1 - ramp)
+
+
+class AngleRotary(nn.Module):
+    """Rotary embedding without a table: fp32 frequencies, the angle position * f_i formed in fp32 inside the kernel,
+    interleaved pairs (2i, 2i+1) of the first ``dims`` coordinates, cos and sin scaled by ``magnitude``.  ``scaling`` =
+    {factor, original, fast, slow} blends the frequencies (yarn_blend) and sets magnitude = 0.1 ln(factor) + 1."""
+
+    def __init__(self, dims: int, base: float, scaling: Optional[Dict[str, Any]] = None) -> None:
+        super().__init__()
+        if dims % 2:
+            raise ValueError("rotary dims must be even")
+        if scaling:
+            freq = yarn_blend(dims, base, scaling["factor"], scaling["original"], scaling["fast"], scaling["slow"])
+            self.magnitude = 0.1 * math.log(scaling["factor"]) + 1.0
+        else:
+            freq = torch.tensor([base ** (-2.0 * i / dims) for i in range(dims // 2)], dtype=torch.float64)
+            self.magnitude = 1.0
+        self.dims = dims
+        self.register_buffer("freq", freq.to(torch.float32), persistent=False)
+
+    def forward(self, positions: torch.Tensor, x: torch.Tensor, offset: int = 0) -> None:
+        """in place on x [T, H, n]: coordinates offset .. offset + dims of every head"""
+        _native.rotary_interleaved(x, positions, self.freq, self.magnitude, offset)

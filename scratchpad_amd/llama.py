@@ -291,7 +291,9 @@ class LogitsProcessor(nn.Module):
         want_input = (fb.forward_mode.is_extend() and fb.return_logprob and fb.extend_logprob_start_lens_cpu is not None
                       and any(e - s > 0 for e, s in zip(fb.extend_seq_lens_cpu, fb.extend_logprob_start_lens_cpu)))
         if not want_input:
-            if fb.forward_mode.is_decode_or_idle():
+            if getattr(fb, "logit_rows", None) is not None:
+                pruned = hidden_states[fb.logit_rows]
+            elif fb.forward_mode.is_decode_or_idle():
                 pruned = hidden_states
             else:
                 last_index = torch.cumsum(fb.extend_seq_lens, dim=0) - 1

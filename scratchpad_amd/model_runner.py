@@ -18,7 +18,8 @@ from .attention import HipAttnBackend
 from .forward_info import CaptureHiddenMode, ForwardBatch, ForwardMode, ModelWorkerBatch
 from .llama import LlamaForCausalLM, LogitsProcessorOutput
 from .sampler import Sampler
-from .pool import MHATokenToKVPool, ReqToTokenPool, TokenToKVPoolAllocator
+from .pool import (LatentTokenToKVPool, MHATokenToKVPool, RecurrentStatePool, ReqToTokenPool,
+                   TokenToKVPoolAllocator)
 
 
 @dataclass
@@ -102,12 +103,14 @@ class ServerArgs:
     kv_cache_dtype: str = "auto"
 
 
-def get_batch_sizes_to_capture(server_args: ServerArgs, max_reqs: int) -> List[int]:
-    """cuda_graph_runner.py:92-128 with the bucket list extended to cuda_graph_max_bs."""
+def get_batch_sizes_to_capture(server_args: ServerArgs, max_reqs: int, model_cap: Optional[int] = None) -> List[int]:
+    """cuda_graph_runner.py:92-128 with the bucket list extended to cuda_graph_max_bs.  ``model_cap``: the largest step a
+    model class allows to be captured (``max_graph_batch``); larger steps run eagerly."""
     bs = server_args.cuda_graph_bs
     if bs is None:
         bs = [1, 2, 4, 8] + list(range(16, server_args.cuda_graph_max_bs + 1, 8))
-    return sorted({b for b in bs if b <= max_reqs and b <= server_args.cuda_graph_max_bs})
+    cap = server_args.cuda_graph_max_bs if model_cap is None else min(server_args.cuda_graph_max_bs, model_cap)
+    return sorted({b for b in bs if b <= max_reqs and b <= cap})
 
 
 class ModelRunner:
@@ -149,16 +152,19 @@ class ModelRunner:
 
     # ------------------------------------------------------------------ model
     def load_model(self, seed: int, init_weights: bool):
+        from .registry import model_class_for
+        model_class = model_class_for(self.model_config)
+        if self.tp_size > 1 and not getattr(model_class, "supports_tensor_parallel", True):
+            raise NotImplementedError(f"{model_class.__name__} is not sharded: run it with tp_size 1")
         with torch.device(self.device):
-            if self.model_config.is_encoder_decoder:
-                from .mllama import MllamaForConditionalGeneration
-                self.model = MllamaForConditionalGeneration(self.model_config, dtype=self.dtype).eval()
-            else:
-                self.model = LlamaForCausalLM(self.model_config, dtype=self.dtype).eval()
-        for p in self.model.parameters():
-            if p.dtype != self.dtype:
-                p.data = p.data.to(self.dtype)
-        if init_weights:
+            self.model = model_class(self.model_config, dtype=self.dtype).eval()
+        if not getattr(model_class, "keeps_parameter_dtypes", False):
+            for p in self.model.parameters():
+                if p.dtype != self.dtype:
+                    p.data = p.data.to(self.dtype)
+        if init_weights and hasattr(self.model, "init_random"):
+            self.model.init_random(torch.Generator(device=self.device).manual_seed(seed + 1000 * self.tp_rank))
+        elif init_weights:
             g = torch.Generator(device=self.device).manual_seed(seed + 1000 * self.tp_rank)
             for name, p in self.model.named_parameters():
                 if "norm" in name:
@@ -172,6 +178,8 @@ class ModelRunner:
     def profile_max_num_token(self) -> int:
         """model_runner.py:325-358: tokens that fit in mem_fraction_static of the free memory."""
         free, _total = torch.cuda.mem_get_info()
+        if hasattr(self.model_config, "cache_bytes_per_token"):
+            return int(free * self.server_args.mem_fraction_static // self.model_config.cache_bytes_per_token(self.kv_cache_dtype))
         cell = (self.model_config.get_num_kv_heads(self.tp_size) * self.model_config.head_dim *
                 self.model_config.num_hidden_layers * 2 * torch.finfo(self.kv_cache_dtype).bits // 8)
         return int(free * self.server_args.mem_fraction_static // cell)
@@ -186,6 +194,19 @@ class ModelRunner:
             max_reqs = min(max(int(self.max_total_num_tokens / self.model_config.context_len * 512),
                                2048), 4096)
         self.max_running_requests = max_reqs
+        self.state_pool = None
+        if hasattr(self.model_config, "latent_cache"):
+            # latent key/value rows for the attention layers, per-request state for the recurrent ones; request row 0 is
+            # kept back for the padded rows of a graph replay (they must not touch a live request's state)
+            self.req_to_token_pool = ReqToTokenPool(max_reqs + 1, self.model_config.context_len + 4, self.device,
+                                                    reserved_rows=1)
+            self.token_to_kv_pool = LatentTokenToKVPool(self.max_total_num_tokens, self.kv_cache_dtype,
+                                                        self.model_config.latent_cache(), self.device)
+            self.state_pool = RecurrentStatePool(max_reqs + 1, self.model_config.hidden_size,
+                                                 self.model_config.recurrent_layers(), self.device)
+            self.token_to_kv_pool_allocator = TokenToKVPoolAllocator(
+                self.max_total_num_tokens, self.kv_cache_dtype, self.device, self.token_to_kv_pool)
+            return
         self.req_to_token_pool = ReqToTokenPool(max_reqs + 1, self.model_config.context_len + 4,
                                                 self.device)
         self.token_to_kv_pool = MHATokenToKVPool(
@@ -198,13 +219,20 @@ class ModelRunner:
     def init_attention_backend(self):
         if self.server_args.attention_backend != "hip":
             raise ValueError(f"Invalid attention backend: {self.server_args.attention_backend}")
-        self.attn_backend = HipAttnBackend(self)
+        if self.state_pool is not None:
+            from .attention import SequenceBackend
+            self.attn_backend = SequenceBackend(self)
+        else:
+            self.attn_backend = HipAttnBackend(self)
         self.sampler = Sampler(tp_group=dist_.get_tp_group())
 
     def init_cuda_graphs(self):
         """model_runner.py:490-504."""
         if self.server_args.disable_cuda_graph:
             return
+        cap = getattr(self.model, "max_graph_batch", None)
+        if cap is not None and not get_batch_sizes_to_capture(self.server_args, self.req_to_token_pool.size, cap):
+            return                      # every requested bucket is above what this model lets into a graph: eager decode
         if _native._LIBROWS_MODE == "auto":
             # SP_LIBRARY_ROWS=auto: measure, on this box and this library build, which graph buckets are
             # cheaper when the library is handed a few more rows (_native.calibrate_library_rows)
@@ -282,8 +310,10 @@ class HipGraphRunner:
         self.model_runner = model_runner
         self.graphs: Dict[int, torch.cuda.CUDAGraph] = {}
         self.output_buffers: Dict[int, LogitsProcessorOutput] = {}
-        self.capture_bs = get_batch_sizes_to_capture(model_runner.server_args,
-                                                     model_runner.req_to_token_pool.size)
+        self.capture_bs = get_batch_sizes_to_capture(model_runner.server_args, model_runner.req_to_token_pool.size,
+                                                     getattr(model_runner.model, "max_graph_batch", None))
+        if not self.capture_bs:
+            raise RuntimeError("no batch size to capture: the model's max_graph_batch is below every requested bucket")
         self.max_bs = max(self.capture_bs)
         backend = model_runner.attn_backend
         backend.init_cuda_graph_state(self.max_bs)
@@ -333,7 +363,7 @@ class HipGraphRunner:
             out_cache_loc=self.out_cache_loc[:bs], seq_lens_sum=int(self.seq_len_fill_value) * bs,
             positions=self.positions[:bs], req_to_token_pool=mr.req_to_token_pool,
             token_to_kv_pool=mr.token_to_kv_pool, attn_backend=mr.attn_backend,
-            capture_hidden_mode=CaptureHiddenMode.NULL)
+            capture_hidden_mode=CaptureHiddenMode.NULL, state_pool=getattr(mr, "state_pool", None))
         enc = None
         if self.is_encoder_decoder:
             enc = self.encoder_lens[:bs]
@@ -372,6 +402,7 @@ class HipGraphRunner:
         if bs != raw_bs:
             self.seq_lens.fill_(self.seq_len_fill_value)
             self.out_cache_loc.zero_()
+            self.req_pool_indices.zero_()      # padded rows write per-request state (if the model has any) to row 0 only
             if self.encoder_lens is not None:
                 self.encoder_lens.zero_()
         if self.encoder_lens is not None:

@@ -66,7 +66,11 @@ class ReqToTokenPool:
     ``write`` and the write journal (``get_write_records`` / ``apply_write_records``, used by the
     reference's overlap worker to mirror table writes).  Rows are handed out first-freed-first."""
 
-    def __init__(self, size: int, max_context_len: int, device: str, use_records: bool = False):
+    def __init__(self, size: int, max_context_len: int, device: str, use_records: bool = False,
+                 reserved_rows: int = 0):
+        # reserved_rows: the first rows are never handed out.  Models with per-request state (RecurrentStatePool) keep
+        # row 0 for the padded rows of a graph replay, which carry request index 0 and must not touch a live state.
+        self.reserved_rows = reserved_rows
         self.size = size
         self.max_context_len = max_context_len
         self.device = device
@@ -97,7 +101,7 @@ class ReqToTokenPool:
         self._rows.push([free_index] if isinstance(free_index, int) else free_index)
 
     def clear(self) -> None:
-        self._rows.load(np.arange(self.size))
+        self._rows.load(np.arange(self.reserved_rows, self.size))
         self._journal = []
 
     def write(self, indices, values) -> None:
@@ -385,3 +389,77 @@ class MHATokenToKVPool(KVCache):
             cache_k = cache_k.to(self.dtype)
             cache_v = cache_v.to(self.dtype)
         _native.kv_store(self.k_buffer[layer_id], self.v_buffer[layer_id], loc, cache_k, cache_v)
+
+
+class LatentTokenToKVPool(KVCache):
+    """Token-level pool of a compressed key/value cache: per layer ONE row per token, ``[normed latent | rotated shared
+    key part]`` - every head's key and value derive from it, so nothing per head is stored.  Same slot ids, allocator
+    and dummy slot 0 as MHATokenToKVPool; only the layers named in ``layers`` ({layer id: (rank, rot_dim)}, each with
+    its own widths) take memory.  ``get_key_buffer`` is the layer's [P+1, rank + rot_dim] buffer; the value is its first
+    ``rank`` columns."""
+
+    def __init__(self, size: int, dtype: torch.dtype, layers, device: str):
+        if dtype not in (torch.float32, torch.float16, torch.bfloat16):
+            raise NotImplementedError(f"latent KV cache dtype {dtype} is not built")
+        self.size, self.page_size, self.dtype, self.store_dtype, self.device = size, 1, dtype, dtype, device
+        self.layers = {int(l): (int(r), int(d)) for l, (r, d) in layers.items()}
+        self._buffers = {l: torch.zeros((size + 1, r + d), dtype=dtype, device=device) for l, (r, d) in self.layers.items()}
+        self.layer_num = len(self.layers)
+        self.layer_transfer_counter = None
+
+    def get_kv_size_bytes(self):
+        return sum(b.nbytes for b in self._buffers.values()), 0
+
+    def get_key_buffer(self, layer_id: int) -> torch.Tensor:
+        return self._buffers[layer_id]
+
+    def get_value_buffer(self, layer_id: int) -> torch.Tensor:
+        return self._buffers[layer_id][:, :self.layers[layer_id][0]]
+
+    def get_kv_buffer(self, layer_id: int):
+        return self.get_key_buffer(layer_id), self.get_value_buffer(layer_id)
+
+    def set_kv_buffer(self, layer, loc: torch.Tensor, cache_k: torch.Tensor, cache_v: torch.Tensor = None) -> None:
+        """rows already normed and rotated (the fused store, _native.latent_kv_store, is what the model path runs)"""
+        self._buffers[layer.layer_id][loc] = cache_k.to(self.dtype)
+
+    def get_flat_data(self, indices):
+        return [self._buffers[l][indices] for l in sorted(self._buffers)]
+
+    def transfer(self, indices, flat_data):
+        for l, data in zip(sorted(self._buffers), flat_data):
+            self._buffers[l][indices] = data.to(device=self.device, non_blocking=False)
+
+    def transfer_per_layer(self, indices, flat_data, layer_id):
+        self._buffers[layer_id][indices] = flat_data.to(device=self.device, non_blocking=False)
+
+
+class RecurrentStatePool:
+    """Per-request state of models whose layers carry something from token to token besides a key/value cache: one slot
+    per row of the ReqToTokenPool (the request's row index IS its state slot, so admission, release and reuse of a slot
+    are the request table's), fp32 throughout.
+
+    * ``last_token`` [slots] int64: the request's latest token (input of a hashed previous-token embedding);
+    * per recurrent layer ``shift`` [slots, width] (the layer input of the latest token, for the token shift) and
+      ``matrix`` [slots, heads, dim, dim] (the recurrence's state);
+    * nothing is cleared when a slot changes hands: every kernel starts a request that holds no token yet from the initial
+      state, whatever the slot contains.  Row 0 belongs to the padded rows of a graph replay (ReqToTokenPool.reserved_rows)."""
+
+    def __init__(self, slots: int, width: int, layers, device: str):
+        """layers: {layer_id: (heads, dim)} of the recurrent layers"""
+        self.slots, self.width, self.device = slots, width, device
+        self.layer_ids = sorted(layers)
+        self._index = {l: i for i, l in enumerate(self.layer_ids)}
+        self.last_token = torch.zeros(slots, dtype=torch.int64, device=device)
+        self.shift = torch.zeros((len(self.layer_ids), slots, width), dtype=torch.float32, device=device)
+        self.matrix = [torch.zeros((slots, h, d, d), dtype=torch.float32, device=device)
+                       for h, d in (layers[l] for l in self.layer_ids)]
+
+    def shift_state(self, layer_id: int) -> torch.Tensor:
+        return self.shift[self._index[layer_id]]
+
+    def matrix_state(self, layer_id: int) -> torch.Tensor:
+        return self.matrix[self._index[layer_id]]
+
+    def size_bytes(self) -> int:
+        return self.last_token.nbytes + self.shift.nbytes + sum(m.nbytes for m in self.matrix)

@@ -99,6 +99,9 @@ class Req:
         self.return_hidden_states = return_hidden_states
         self.topping_path = topping_path
         self.req_pool_idx: Optional[int] = None
+        # True: the request keeps its row of the request table (and with it its state slot, for models with per-request
+        # state) from one extend step to the next; prepare_for_extend then allocates no new row for it
+        self.keeps_pool_row = False
         # finishing (check_finished)
         self.tokenizer = None
         self.finished_reason = None
@@ -210,6 +213,7 @@ class Req:
         self.fill_ids_override = None
         self.extend_input_len_override = None
         self.req_pool_idx = None
+        self.keeps_pool_row = False
         self.extend_logprob_start_len = 0
         self.is_retracted = True
         self.is_chunked = 0
@@ -341,7 +345,8 @@ class ScheduleBatch:
         self.forward_mode = ForwardMode.EXTEND
         reqs = self.reqs
         bs = len(reqs)
-        req_pool_indices = self.alloc_req_slots(bs)
+        fresh = iter(self.alloc_req_slots(sum(1 for r in reqs if not (r.keeps_pool_row and r.req_pool_idx is not None))))
+        req_pool_indices = [r.req_pool_idx if r.keeps_pool_row and r.req_pool_idx is not None else next(fresh) for r in reqs]
         input_ids = [r.fill_ids[r.prefix_len:] for r in reqs]
         extend_num_tokens = sum(len(ids) for ids in input_ids)
         seq_lens = [len(r.fill_ids) for r in reqs]
