@@ -70,9 +70,16 @@ def parse_args():
     ap.add_argument("--sample", action="store_true",
                     help="serve mode: temperature 0.8 / top-p 0.9 / top-k 50 sampling instead of greedy")
     ap.add_argument("--rate", type=float, default=0.0, help="serve mode: Poisson arrival rate (req/s); 0 = all at t=0")
-    ap.add_argument("--mode", default="decode", choices=["decode", "prefill", "serve", "tp"],
+    ap.add_argument("--mode", default="decode", choices=["decode", "prefill", "serve", "tp", "hybrid"],
                     help="decode = the headline metric (+ the TTFT half); prefill = config 3 alone; "
-                         "tp = config 4 (sharded model, RCCL)")
+                         "tp = config 4 (sharded model, RCCL); hybrid = the Tizalorn design (recurrent + latent-attention "
+                         "+ expert layers) beside a Llama of equal width and depth, with a per-kernel roofline table "
+                         "(bench_hybrid.py)")
+    ap.add_argument("--sizes", default="l", help="hybrid mode: model widths to run, of m (2048) and l (4096)")
+    ap.add_argument("--no-kernel-table", action="store_true", help="hybrid mode: throughput only")
+    ap.add_argument("--graph", action="store_true",
+                    help="hybrid mode: replay captured decode steps (default: eager launches for both models; a model class "
+                         "may cap the step size it lets into a graph)")
     ap.add_argument("--no-ttft", action="store_true", help="decode mode: skip the config-3 TTFT passes")
     ap.add_argument("--prefix", type=int, default=0, help="prefill mode: shared cached prefix length")
     ap.add_argument("--max-prefill-tokens", type=int, default=16384,
@@ -883,6 +890,12 @@ def tp_main(args, rank, local_rank, world):
 
 def main():
     args = parse_args()
+    if args.mode == "hybrid":              # (a parent of one child process per model: nothing here touches the GPU)
+        if args.gpus != 1:
+            raise SystemExit("--mode hybrid is a one-GPU comparison")
+        from bench_hybrid import hybrid_main
+        hybrid_main(args)
+        return
     self_launch_if_needed(args)
     rank = int(os.environ.get("RANK", "0"))
     local_rank = int(os.environ.get("LOCAL_RANK", "0"))

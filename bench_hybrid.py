@@ -1,0 +1,308 @@
+"""bench.py --mode hybrid: prefill and decode throughput of the Tizalorn design at layer sizes of real models (random
+weights), beside a Llama of the same width and depth on the same engine path, and a per-kernel table: every HIP kernel
+(and library product) of both models timed inside an eager prefill batch and an eager decode step, with the time its
+algorithmic bytes and flops would take at the chip's peaks (fraction of roofline).
+
+Workload per size: `bs` requests of `ctx` prompt tokens, prefilled through ScheduleBatch.prepare_for_extend in extend
+batches of at most --max-prefill-tokens tokens, then --steps decode steps (HIP-graph replay unless --no-graph) feeding
+the sampled tokens back.  One JSON line per run; the default bench.py workload and its line are untouched."""
+import json
+import time
+
+import torch
+
+HBM = 8.0e12            # bytes/s
+MATRIX = 2.5e15         # dense bf16 flops/s on the matrix cores
+VECTOR32 = 157.3e12     # fp32 flops/s on the vector units (kernels whose arithmetic is fp32 by contract)
+
+SIZES = {"m": 2048, "l": 4096}      # widths of Llama-3.2-1B and Llama-3-8B, whose layers are the comparison
+# Decode steps are launched eagerly for both models unless --graph is given.
+
+
+def tizalorn_config(width: int, layers: int, context_len: int):
+    from scratchpad_amd.tizalorn import TizalornConfig
+    wkv = {"type": "wkv", "mixer": {"heads": width // 64, "dim": 64, "decay_rank": 64}}
+    lat = {"type": "latent_attention",
+           "mixer": {"heads": width // 128, "dim": 128, "rot_dim": 64, "vdim": 128, "kv_rank": 512, "q_rank": 3 * width // 4,
+                     "rot": {"base": 50000.0, "dims": 64, "scaling": {"factor": 8.0, "original": 4096, "fast": 16.0, "slow": 2.0}},
+                     "scale": 192 ** -0.5}}
+    dense = {"kind": "dense", "ff": {2048: 8192, 4096: 14336}.get(width, 3 * width)}
+    moe = {"kind": "moe", "expert": {"ff": width // 2, "limit": 7.0},
+           "router": {"experts": 32, "top": 4, "groups": {"count": 4, "keep": 2}}}
+    pattern = [(wkv, dense), (wkv, moe), (lat, moe), (wkv, moe)]
+    raw = {"architecture": "Tizalorn", "vocab": 128256, "width": width, "norm": {"eps": 1e-5},
+           "embedding": {"bigram": {"buckets": 65521, "mul_prev": 131, "mul_cur": 31}},
+           "layers": [{**pattern[i % 4][0], "mlp": pattern[i % 4][1]} for i in range(layers)]}
+    return TizalornConfig(raw, context_len=context_len)
+
+
+def llama_config(width: int, layers: int, context_len: int):
+    """the layers of Llama-3.2-1B (width 2048) / Llama-3-8B (width 4096), `layers` of them"""
+    from scratchpad_amd.model_runner import ModelConfig
+    cfg = {2048: ModelConfig.llama32_1b, 4096: ModelConfig.llama3_8b}[width](context_len)
+    cfg.num_hidden_layers = layers
+    return cfg
+
+
+def say(*what):
+    print("[hybrid]", *what, flush=True)
+
+
+# ----------------------------------------------------------------------------------------------- per-kernel accounting
+def _nbytes(*ts):
+    return sum(t.numel() * t.element_size() for t in ts if isinstance(t, torch.Tensor))
+
+
+class KernelClock:
+    """wraps functions of scratchpad_amd._native (and the library products the models call) with HIP events"""
+
+    def __init__(self):
+        self.rows = {}          # name -> [events, bytes, flops, peak]
+        self.step = None        # {"prefix": [...], "extend": [...]} of the running step, for the attention costs
+
+    def pairs(self):
+        """(query, visible key) pairs of the step"""
+        return sum(e * p + e * (e + 1) // 2 for p, e in zip(self.step["prefix"], self.step["extend"]))
+
+    def keys_read(self):
+        return sum(p + e for p, e in zip(self.step["prefix"], self.step["extend"]))
+
+    def record(self, name, fn, cost):
+        def timed(*a, **k):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            out = fn(*a, **k)
+            e1.record()
+            b, f, peak = cost(a, k, out)
+            row = self.rows.setdefault(name, [[], 0, 0, peak])
+            row[0].append((e0, e1))
+            row[1] += b
+            row[2] += f
+            return out
+        return timed
+
+    def table(self):
+        torch.cuda.synchronize()
+        out = []
+        for name, (events, b, f, peak) in self.rows.items():
+            ms = sum(a.elapsed_time(z) for a, z in events)
+            roof_ms = max(b / HBM, f / peak) * 1e3
+            out.append({"kernel": name, "calls": len(events), "ms": round(ms, 4), "bound": "hbm" if b / HBM >= f / peak else "flops",
+                        "roofline_ms": round(roof_ms, 4), "frac": round(roof_ms / ms, 4) if ms > 0 else None})
+        return sorted(out, key=lambda r: -r["ms"])
+
+
+def instrument(clock: KernelClock, cfg):
+    """patch the kernels' Python entry points; returns the undo function"""
+    from scratchpad_amd import _native as N
+    saved = {}
+
+    def io(a, k, out):           # elementwise / row kernels: every tensor argument and result once
+        outs = out if isinstance(out, (tuple, list)) else (out,)
+        return _nbytes(*a, *k.values(), *outs), 0, MATRIX
+
+    def gemm(a, k, out):
+        x, w = a[0], a[1]
+        return _nbytes(x, w, out), 2 * x.shape[0] * w.shape[0] * w.shape[1], MATRIX
+
+    def grouped(a, k, out):
+        x, w = a[0], a[1]
+        E, n, kk = w.shape
+        pairs = a[3]
+        return _nbytes(x, out) + min(E, pairs) * n * kk * w.element_size(), 2 * pairs * n * kk, MATRIX
+
+    def wkv(a, k, out):
+        r, state, heads, dim = a[0], a[7], a[9], a[10]
+        T, live = r.shape[0], len(clock.step["extend"])
+        return _nbytes(*a[:5], out) + 2 * live * heads * dim * dim * 4, 6 * T * heads * dim * dim, VECTOR32
+
+    def latent(a, k, out):
+        q_lat, q_rot, pool = a[0], a[1], a[2]
+        H, T, C = q_lat.shape
+        R = q_rot.shape[2]
+        return _nbytes(q_lat, out) + clock.keys_read() * (C + R) * pool.element_size(), 2 * H * clock.pairs() * (2 * C + R), MATRIX
+
+    def llama_extend(a, k, out):
+        o, q, kb = a[0], a[1], a[2]
+        H, D, Hkv = q.shape[1], q.shape[2], kb.shape[1]
+        return _nbytes(o, q) + clock.keys_read() * 2 * Hkv * D * kb.element_size(), 4 * H * D * clock.pairs(), MATRIX
+
+    costs = {"embed_bigram_norm": io, "add_scalar_norm": io, "scalar_norm": io, "polynorm": io, "gate_heads": io,
+             "token_shift": io, "wkv_decay": io, "wkv_recurrence": wkv, "rotary_interleaved": io, "latent_kv_store": io,
+             "latent_attention": latent, "moe_route": io, "moe_align": io, "moe_grouped_gemm": grouped, "moe_glu": io,
+             "moe_combine": io, "rmsnorm": io, "fused_add_rmsnorm": io, "silu_and_mul": io, "rotary_embedding": io,
+             "extend_attention": llama_extend, "decode_attention": llama_extend, "linear": gemm, "linear_silu_mul": gemm}
+    for name, cost in costs.items():
+        saved[name] = getattr(N, name)
+        setattr(N, name, clock.record(name, saved[name], cost))
+    saved_bmm = torch.bmm
+    torch.bmm = clock.record("bmm (library)", saved_bmm, lambda a, k, out: (
+        _nbytes(a[0], a[1], out), 2 * a[0].shape[0] * a[0].shape[1] * a[0].shape[2] * a[1].shape[2], MATRIX))
+
+    def undo():
+        for name, fn in saved.items():
+            setattr(N, name, fn)
+        torch.bmm = saved_bmm
+    return undo
+
+
+# ----------------------------------------------------------------------------------------------- one model, one size
+def run_model(cfg, args, kernels: bool):
+    from scratchpad_amd.model_runner import ModelRunner, ServerArgs, TpModelWorker
+    from scratchpad_amd.radix_cache import ChunkCache
+    from scratchpad_amd.schedule_batch import Req, ScheduleBatch
+    bs, ctx, steps, warm = args.bs, int(args.ctx), args.steps, args.warmup
+    pool_tokens = bs * (ctx + 2 * (steps + warm) + 8) + 64
+    sargs = ServerArgs(max_total_tokens=pool_tokens, max_running_requests=bs, disable_cuda_graph=args.no_graph,
+                       cuda_graph_max_bs=bs, cuda_graph_bs=[bs])
+    name = type(cfg).__name__
+    say(name, "width", cfg.hidden_size, ": building the runner")
+    mr = ModelRunner(cfg, sargs, dtype=torch.bfloat16, seed=0)
+    worker = TpModelWorker(mr)
+    if not args.no_graph:
+        say(name, ": capturing the decode graph, bs", bs)
+        mr.init_cuda_graphs()
+    cache = ChunkCache(mr.req_to_token_pool, token_to_kv_pool_allocator=mr.token_to_kv_pool_allocator)
+    gen = torch.Generator().manual_seed(0)
+    clock = KernelClock()
+
+    def prefill(tag):
+        reqs = [Req(f"{tag}{i}", "", torch.randint(0, cfg.vocab_size, (ctx,), generator=gen).tolist(), None) for i in range(bs)]
+        per = max(1, args.max_prefill_tokens // ctx)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        batches = []
+        for lo in range(0, bs, per):
+            b = ScheduleBatch(reqs[lo:lo + per], mr.req_to_token_pool, mr.token_to_kv_pool_allocator, tree_cache=cache,
+                              model_config=cfg, device=mr.device)
+            b.prepare_for_extend()
+            clock.step = {"prefix": b.prefix_lens, "extend": b.extend_lens}
+            _, nxt = worker.forward_batch_generation(b.get_model_worker_batch())
+            b.output_ids = nxt
+            batches.append(b)
+        torch.cuda.synchronize()
+        return reqs, batches, time.perf_counter() - t0
+
+    def release(reqs):
+        for r in reqs:
+            cache.cache_finished_req(r, token_ids=list(r.origin_input_ids))
+
+    say(name, ": warm prefill pass,", bs, "x", ctx, "tokens")
+    reqs, _, _ = prefill("w")                                   # warm pass
+    release(reqs)
+    say(name, ": timed prefill pass")
+    reqs, batches, prefill_s = prefill("p")
+    batch = batches[0]
+    for other in batches[1:]:
+        batch.merge_batch(other)
+
+    def decode(n):
+        for _ in range(n):
+            batch.prepare_for_decode()
+            clock.step = {"prefix": [ctx] * bs, "extend": [1] * bs}
+            _, nxt = worker.forward_batch_generation(batch.get_model_worker_batch())
+            batch.output_ids = nxt
+    say(name, ": decode,", warm, "+", steps, "steps")
+    decode(warm)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    decode(steps)
+    torch.cuda.synchronize()
+    decode_s = time.perf_counter() - t0
+    out = {"prefill_tokens_per_sec": round(bs * ctx / prefill_s, 1), "prefill_ms": round(prefill_s * 1e3, 2),
+           "decode_tokens_per_sec": round(bs * steps / decode_s, 1), "decode_ms_per_step": round(decode_s / steps * 1e3, 3),
+           "parameters": sum(p.numel() for p in mr.model.parameters())}
+    if kernels:
+        graph, mr.graph_runner = mr.graph_runner, None
+        undo = instrument(clock, cfg)
+        try:
+            say(name, ": eager decode step and prefill pass with an event pair around every kernel")
+            decode(1)
+            out["decode_kernels"] = clock.table()
+            clock.rows = {}
+            release(reqs)
+            reqs, _, _ = prefill("k")
+            out["prefill_kernels"] = clock.table()
+        finally:
+            undo()
+            mr.graph_runner = graph
+    release(reqs)
+    del mr, worker
+    torch.cuda.empty_cache()
+    return out
+
+
+DISABLED = ("bench.py --mode hybrid is switched off: its whole-model pass at these layer sizes (8192 and 16384 prompt tokens "
+            "per extend batch, widths 1024 / 2048 / 4096, graph replay and eager) ended the GPU box three times without a "
+            "message, and the cause has not been found - every kernel of the design passes at the same sizes on its own "
+            "(tests/test_gpu_tizalorn_kernels.py).  It stays off the GPU until the cause is shown; see DESIGN.md.")
+
+
+def hybrid_main(args):
+    """the parent: never touches the GPU; one child process per (model, size), so that neither model's graphs, pools or
+    library workspaces are in the other's process"""
+    raise SystemExit(DISABLED)
+    import argparse
+    import os
+    import subprocess
+    import sys
+    widths = [SIZES[s] for s in args.sizes.split(",")]
+    if args.bs == 256:
+        args.bs = 16
+    if args.ctx == "uniform":
+        args.ctx = "1024"
+    if args.steps == 64:
+        args.steps, args.warmup = 32, 4
+    layers = args.layers or 4
+    args.no_graph = not args.graph
+    runs = []
+    for w in widths:
+        row = {"width": w, "layers": layers}
+        for model in ("tizalorn", "llama"):
+            cmd = [sys.executable, "-u", os.path.abspath(__file__), "--child", model, "--width", str(w), "--layers", str(layers),
+                   "--bs", str(args.bs), "--ctx", str(args.ctx), "--steps", str(args.steps), "--warmup", str(args.warmup),
+                   "--max-prefill-tokens", str(args.max_prefill_tokens)]
+            cmd += ["--no-graph"] if args.no_graph else []
+            cmd += ["--no-kernel-table"] if args.no_kernel_table else []
+            say("starting", " ".join(cmd[3:]))
+            p = subprocess.run(cmd, stdout=subprocess.PIPE, text=True)
+            lines = [l for l in p.stdout.splitlines() if l.startswith("RESULT ")]
+            sys.stdout.write("".join(l + "\n" for l in p.stdout.splitlines() if not l.startswith("RESULT ")))
+            if p.returncode != 0 or not lines:
+                raise SystemExit(f"{model} at width {w} failed (exit code {p.returncode})")
+            row[model] = json.loads(lines[-1][len("RESULT "):])
+            say(model, "width", w, {k: v for k, v in row[model].items() if "kernels" not in k})
+        runs.append(row)
+    last = runs[-1]
+    print(json.dumps({
+        "metric": "hybrid_decode_tokens_per_sec", "value": last["tizalorn"]["decode_tokens_per_sec"], "unit": "tokens/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": last["tizalorn"]["decode_ms_per_step"],
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+        "data": "synthetic (random-init weights, random prompts)",
+        "config": {"workload": f"Tizalorn vs Llama layers at equal width and depth, bs={args.bs} prompts of {args.ctx} tokens, "
+                               f"extend batches <= {args.max_prefill_tokens} tokens, then {args.steps} decode steps, "
+                               f"{'eager' if args.no_graph else 'HIP-graph replay'}", "sizes": runs}}), flush=True)
+
+
+def child_main():
+    raise SystemExit(DISABLED)
+    import argparse
+    import os
+    import sys
+    sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--child", required=True, choices=["tizalorn", "llama"])
+    for name in ("width", "layers", "bs", "ctx", "steps", "warmup", "max-prefill-tokens"):
+        ap.add_argument("--" + name, type=int, required=True)
+    ap.add_argument("--no-graph", action="store_true")
+    ap.add_argument("--no-kernel-table", action="store_true")
+    a = ap.parse_args()
+    torch.cuda.set_device(0)
+    ctx_len = a.ctx + 2 * (a.steps + a.warmup) + 16
+    cfg = (tizalorn_config if a.child == "tizalorn" else llama_config)(a.width, a.layers, ctx_len)
+    out = run_model(cfg, a, not a.no_kernel_table)
+    print("RESULT " + json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    child_main()
