@@ -235,7 +235,7 @@ def run_model(cfg, args, kernels: bool):
 DISABLED = ("bench.py --mode hybrid is switched off: its whole-model pass at these layer sizes (8192 and 16384 prompt tokens "
             "per extend batch, widths 1024 / 2048 / 4096, graph replay and eager) ended the GPU box three times without a "
             "message, and the cause has not been found - every kernel of the design passes at the same sizes on its own "
-            "(tests/test_gpu_tizalorn_kernels.py).  It stays off the GPU until the cause is shown; see DESIGN.md.")
+            "(tests/test_gpu_tizalorn_kernels.py).  It stays off the GPU until the cause is shown.")
 
 
 def hybrid_main(args):
