@@ -62,23 +62,6 @@ def _w64_asm():
     return w64_asm
 
 
-def check_w64_descriptors(lib: str = LIB, verbose: bool = False) -> None:
-    """Raise unless the library's extend_w64 kernels carry what this source tree expects (tools/w64_asm.py check):
-    kernel descriptor == .amdgpu_metadata note == ACCUM_OFFSET + 256 registers of which 256 accumulation, and the host
-    flag the launcher checks is 1.  A library linked from a plain `hipcc -c extend_w64.hip`, or compiled by a toolchain
-    that lays the kernels' registers out differently, fails the BUILD, not a parity test on a GPU box."""
-    import contextlib
-    import io
-    buf = io.StringIO()
-    with contextlib.redirect_stdout(buf):
-        ok = _w64_asm().check(lib)
-    if verbose or not ok:
-        print(buf.getvalue(), end="")
-    if not ok:
-        raise RuntimeError(f"{lib}: the extend_w64 kernel descriptors are not what extend_w64.hip needs (see above); "
-                           "rebuild with `python -m scratchpad_amd.build --force`")
-
-
 def compile_w64(src: str, obj: str, extra=(), verbose: bool = True) -> str:
     """extend_w64.hip in stages, so that the accumulation registers only its asm text names are allocated where the
     ASSEMBLER can see and validate them (until round 4 the linked .so was byte-patched):
@@ -136,7 +119,6 @@ def build_native(force: bool = False, verbose: bool = True, only=None) -> str:
             srcs = [x for x in srcs if os.path.basename(x) in have]      # up to date? checked below against ITS sources
         else:
             srcs = [x for x in srcs if os.path.basename(x) in want]
-    partial = not any(os.path.basename(x) == "extend_w64.hip" for x in srcs)
     hdrs = sorted(glob.glob(os.path.join(CSRC, "*.h"))) + sorted(glob.glob(os.path.join(CSRC, "*.inc"))) + [
         os.path.join(ROOT, "include", "scratchpad_hip.h"), os.path.join(ROOT, "tools", "w64_asm.py")]
     # (the library also has to be made of exactly these sources and flags: a source removed - or a flag changed - leaves
@@ -147,8 +129,6 @@ def build_native(force: bool = False, verbose: bool = True, only=None) -> str:
                         ["compiler: " + _hipcc_version()])
     same = os.path.exists(stamp) and open(stamp).read() == made_of
     if not force and same and _newer(LIB, srcs + hdrs):
-        if not partial:
-            check_w64_descriptors(LIB)   # (cheap: reads the ELF; a library somebody linked by hand fails here)
         return LIB
     force = force or not same
     os.makedirs(OBJ, exist_ok=True)
@@ -172,8 +152,6 @@ def build_native(force: bool = False, verbose: bool = True, only=None) -> str:
     if verbose:
         print(" ".join(cmd), flush=True)
     subprocess.run(cmd, check=True)
-    if not partial:
-        check_w64_descriptors(LIB, verbose)
     with open(stamp, "w") as f:
         f.write(made_of)
     return LIB

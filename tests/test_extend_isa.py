@@ -59,7 +59,6 @@ def test_tile_loop_keeps_its_dma_in_flight(dma_kernel_asm):
 # scratch in the tile loop (its wait drains the DMA ring), the generated bodies drifting away from their generator.
 W64_FLAGS = ["-fno-honor-nans", "-fno-slp-vectorize", "-std=c++20", "-mllvm", "-amdgpu-atomic-optimizer-strategy=None"]
 LIB = os.path.join(ROOT, "scratchpad_amd", "lib", "libscratchpad_hip.so")
-READELF = "/opt/rocm/lib/llvm/bin/llvm-readelf"
 
 
 def _w64_tool():
@@ -80,46 +79,6 @@ def test_w64_generated_bodies_are_the_generators_output():
 def test_w64_build_flags_are_the_tested_ones():
     from scratchpad_amd import build
     assert build.PER_FILE_FLAGS["extend_w64.hip"] == W64_FLAGS
-
-
-def test_built_library_gives_the_w64_kernels_their_accumulation_registers():
-    if not os.path.exists(LIB):
-        pytest.skip("library not built")
-    r = subprocess.run(["python3", os.path.join(ROOT, "tools", "w64_asm.py"), "check", LIB], capture_output=True, text=True)
-    assert r.returncode == 0 and r.stdout.count("-> ok") == 4 and "sp_w64_descriptor_patched = 1" in r.stdout, r.stdout + r.stderr
-    # and a library linked WITHOUT the staged build refuses to launch them: the flag the kernel's host side checks is not 1
-    import ctypes
-    assert ctypes.c_int.in_dll(ctypes.CDLL(LIB), "sp_w64_descriptor_patched").value == 1
-
-
-def test_shipped_code_object_is_self_consistent(tmp_path):
-    """VERDICT r4 item 4, checked with the toolchain's own reader rather than this repo's ELF walker: `llvm-readelf
-    --notes` on the w64 code object extracted from the shipped library reports agpr_count 256 and vgpr_count =
-    ACCUM_OFFSET + 256 for the four kernels, and the kernel descriptors (read from .rodata) allocate exactly that."""
-    import struct
-    if not os.path.exists(LIB) or not os.path.exists(READELF):
-        pytest.skip("library or llvm-readelf not available")
-    w = _w64_tool()
-    data = open(LIB, "rb").read()
-    hits = 0
-    for base, size in w.device_elves(data):
-        descs = dict(w.descriptors(data, base))
-        if not descs:
-            continue
-        co = tmp_path / "w64.hsaco"
-        co.write_bytes(data[base:base + size])
-        txt = subprocess.run([READELF, "--notes", str(co)], check=True, capture_output=True, text=True).stdout
-        for name, off in descs.items():
-            entry = re.search(r"- \.agpr_count:\s+(\d+)\n(?:(?!- \.agpr_count).)*?\n\s+\.name:\s+" + re.escape(name) +
-                              r"\n(?:(?!- \.agpr_count).)*?\.vgpr_count:\s+(\d+)", txt, re.S)
-            assert entry, name
-            agpr, vgpr = int(entry.group(1)), int(entry.group(2))
-            rsrc3, rsrc1 = struct.unpack_from("<II", data, off + 44)
-            accum, regs = ((rsrc3 & 0x3F) + 1) * 4, ((rsrc1 & 0x3F) + 1) * 8
-            assert agpr == 256 and vgpr == accum + 256 == w.EXPECTED[w.kernel_of(name)] + 256, (name, agpr, vgpr, accum)
-            assert regs == (vgpr + 7) // 8 * 8, (name, regs, vgpr)
-            hits += 1
-    assert hits == 4
 
 
 def test_w64_rewrite_refuses_a_different_register_layout():
@@ -147,42 +106,6 @@ def test_w64_rewrite_refuses_a_different_register_layout():
         w.rewrite(text([good[0] - 4] + good[1:]))
     with pytest.raises(SystemExit, match="allocates accumulation registers"):
         w.rewrite(text(good).replace(f".amdhsa_next_free_vgpr {good[0] - 1}\n", f".amdhsa_next_free_vgpr {good[0] + 8}\n", 1))
-
-
-def test_build_refuses_an_unstaged_or_differently_laid_out_library(tmp_path):
-    """the register allocation of the w64 kernels must fail at BUILD time.  build_native() ends with
-    check_w64_descriptors(); a copy of the library whose descriptor no longer matches its note (register granules back to
-    what hipcc would have written), whose host flag is cleared (what a plain `hipcc -c extend_w64.hip` links), or whose
-    ACCUM_OFFSET is not the one the kernels' text assumes, is refused."""
-    import shutil
-    import struct
-    from scratchpad_amd import build
-    if not os.path.exists(LIB):
-        pytest.skip("library not built")
-    build.check_w64_descriptors(LIB)                                   # the shipped library passes
-    assert "compiler: " in open(LIB + ".sources").read(), "the build records hipcc --version next to the library"
-    pw = _w64_tool()
-    data = bytearray(open(LIB, "rb").read())
-    descs = [off for base, _ in pw.device_elves(bytes(data)) for _name, off in pw.descriptors(bytes(data), base)]
-    descs = sorted(set(descs))            # (symtab and dynsym list the same descriptors)
-    assert len(descs) == 4
-    # (1) granule count of one kernel back to 32 granules = 256 registers, what the compiler believes it uses
-    broken = bytearray(data)
-    rsrc1, = struct.unpack_from("<I", broken, descs[0] + 48)
-    struct.pack_into("<I", broken, descs[0] + 48, (rsrc1 & ~0x3F) | 31)
-    # (2) the host flag cleared, descriptors intact
-    noflag = bytearray(data)
-    struct.pack_into("<i", noflag, pw.host_flag_offset(bytes(data)), 2)
-    # (3) another ACCUM_OFFSET (as a different register allocation would give)
-    moved = bytearray(data)
-    rsrc3, = struct.unpack_from("<I", moved, descs[0] + 44)
-    struct.pack_into("<I", moved, descs[0] + 44, (rsrc3 & ~0x3F) | ((rsrc3 & 0x3F) - 2))
-    for name, blob in (("granules", broken), ("flag", noflag), ("accum_offset", moved)):
-        path = tmp_path / f"lib_{name}.so"
-        path.write_bytes(bytes(blob))
-        with pytest.raises(RuntimeError, match="extend_w64 kernel descriptors"):
-            build.check_w64_descriptors(str(path))
-    shutil.rmtree(tmp_path, ignore_errors=True)
 
 
 @pytest.fixture(scope="module")

@@ -10,5 +10,4 @@ mkdir -p build/variants
 python3 -m scratchpad_amd.build --w64-object build/variants/extend_w64_$NAME.o "$@" > /dev/null
 OBJS=$(ls build/obj/*.o | grep -v extend_w64.o)
 /opt/rocm/bin/hipcc --offload-arch=gfx950 -shared -fPIC -o scratchpad_amd/lib/libscratchpad_hip_$NAME.so $OBJS build/variants/extend_w64_$NAME.o
-python3 tools/w64_asm.py check scratchpad_amd/lib/libscratchpad_hip_$NAME.so
 echo built scratchpad_amd/lib/libscratchpad_hip_$NAME.so
