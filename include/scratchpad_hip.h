@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define SP_ABI_VERSION 10
+#define SP_ABI_VERSION 11
 #define SP_API __attribute__((visibility("default")))
 
 typedef enum { SP_F32 = 0, SP_F16 = 1, SP_BF16 = 2, SP_FP8_E5M2 = 3 /* KV pool only */ } sp_dtype;
@@ -480,6 +480,82 @@ SP_API int sp_moe_glu(void* out, const void* gu, int64_t pairs, int ff, float li
 /* out[t] = sum over k < top, in that order, of weights[t, k] * z[place[t * top + k]] */
 SP_API int sp_moe_combine(void* out, const void* z, const int32_t* place, const float* weights, int64_t num_tokens,
                           int width, int top, int64_t out_stride, int dtype, void* stream);
+
+/* Router with softmax scores: z = router x in fp32, s = softmax(z) over all experts; ids [T, top] = the experts with the
+ * largest s (ties: the lower index), weights [T, top] = their s times scale, not renormalised.                      */
+SP_API int sp_moe_route_softmax(int32_t* ids, float* weights, const void* x, int64_t x_stride, const float* router,
+                                int64_t num_tokens, int width, int experts, int top, float scale, int dtype, void* stream);
+
+/* ---- fp32 residual stream of parallel-sublayer layers (csrc/stream_norm.hip) ------------------------------------- */
+/* x[t] = embed[ids[t]] * scale  (x fp32, embed in `dtype`) */
+SP_API int sp_embed_scale(float* x, int64_t x_stride, const void* embed, const int64_t* ids, int64_t num_tokens, int width,
+                          int64_t vocab, float scale, int dtype, void* stream);
+/* h[t] = x[t] / sqrt(mean(x[t]^2) + eps) * weight -> out_h; hs[t] = h[t] + (h[t-1] - h[t]) * mu -> out_hs (both in
+ * `dtype`, either may be null; out_hs null: a plain weighted norm, the request description is not read).  The row before
+ * a step's first row is state[request slot] (zeros at a sequence's first token).                                    */
+SP_API int sp_norm_shift(void* out_h, void* out_hs, int64_t out_stride, const float* x, int64_t x_stride,
+                         const float* weight, const float* mu, const float* state, int64_t state_stride, int64_t num_tokens,
+                         int width, float eps, SP_SEQ_PARAMS, int dtype, void* stream);
+/* state[request slot] = the weighted norm of x[the request's last row of this step]; run after sp_norm_shift */
+SP_API int sp_norm_save_last(float* state, int64_t state_stride, const float* x, int64_t x_stride, const float* weight,
+                             int width, float eps, SP_SEQ_PARAMS, void* stream);
+/* x[t] += a[t] + b[t] + c[t] in fp32 (b, c optional; a, b, c in `dtype`) */
+SP_API int sp_stream_add(float* x, int64_t x_stride, const void* a, int64_t a_stride, const void* b, int64_t b_stride,
+                         const void* c, int64_t c_stride, int64_t num_tokens, int width, int dtype, void* stream);
+
+/* ---- sliding-window attention with pooled blocks (csrc/window_attention.hip) -------------------------------------- */
+/* q [T, heads, dim] rotated in place; k [T, kv_heads, dim] rotated into kpool[loc[t]]; v [T, kv_heads, vdim], every head
+ * divided by its root mean square (eps inside the root), into vpool[loc[t]].  Rotation: coordinate i < rot_dims / 2 pairs
+ * with i + rot_dims / 2, angle = positions[t] * freq[i] in fp32, cos and sin times mag.                              */
+SP_API int sp_qkv_rotary_store(void* q, int64_t q_stride, const void* k, int64_t k_stride, const void* v, int64_t v_stride,
+                               void* kpool, int64_t kp_stride, void* vpool, int64_t vp_stride, const int64_t* positions,
+                               const int64_t* loc, const float* freq, float mag, int64_t num_tokens, int heads, int kv_heads,
+                               int dim, int vdim, int rot_dims, float eps, int dtype, void* stream);
+/* every token of the step whose position + 1 is a multiple of `block` writes the mean of the last `block` cached key rows
+ * (value rows) of its request into kpooled (vpooled) at its own slot; run after the step's rows are in the pool       */
+SP_API int sp_pool_blocks(void* kpooled, void* vpooled, const void* kpool, const void* vpool, int64_t kp_stride,
+                          int64_t vp_stride, const int32_t* req_to_token, int64_t table_stride, int64_t num_tokens,
+                          int key_width, int value_width, int block, SP_SEQ_PARAMS, int dtype, void* stream);
+/* out [T, heads, vdim]: a query at position p attends, in one fp32 softmax of (q . k) * scale, to the cached tokens j with
+ * 0 <= p - j < window and to the pooled rows of the blocks b with b * block + block - 1 <= p - window.  window <= 0: every
+ * earlier token and no blocks; block <= 0: no blocks.  Query head h reads key/value head h / (heads / kv_heads).
+ * vdim <= 256.                                                                                                        */
+SP_API int sp_window_attention(void* out, int64_t out_stride, const void* q, int64_t q_stride, const void* kpool,
+                               const void* vpool, const void* kpooled, const void* vpooled, int64_t kp_stride,
+                               int64_t vp_stride, const int32_t* req_to_token, int64_t table_stride, int64_t num_tokens,
+                               int heads, int kv_heads, int dim, int vdim, int64_t window, int block, float scale,
+                               SP_SEQ_PARAMS, int dtype, void* stream);
+
+/* ---- state-space and matrix-memory recurrences (csrc/ssm.hip, csrc/mlstm.hip) -------------------------------------- */
+/* out[t, j] = bias[j] + sum_i weight[j, i] x[t, i]: fp32 weights, accumulation and output (x in `dtype`; bias optional) */
+SP_API int sp_small_linear_f32(float* out, const void* x, int64_t x_stride, const float* weight, const float* bias,
+                               int64_t num_tokens, int k, int n, int dtype, void* stream);
+/* out[t, c] = silu(bias[c] + sum_j weight[c, j] in[t - (taps - 1) + j, c]); rows before a step's first row come from
+ * state[request slot] ([taps - 1, channels] fp32: the request's latest inputs; zeros before a sequence's start), which is
+ * then moved on to the step's end.  taps <= 16.                                                                      */
+SP_API int sp_causal_conv_silu(void* out, int64_t out_stride, const void* in, int64_t in_stride, const float* weight,
+                               const float* bias, float* state, int64_t state_stride, int64_t num_tokens, int channels,
+                               int taps, SP_SEQ_PARAMS, int dtype, void* stream);
+/* Per (request, head) over the request's rows in order, S [state_size, vdim] fp32 from state[request slot] and back:
+ *   dt = softplus(dt_raw[t, h] + dt_bias[h]); S = exp(-exp(A_log[h]) dt) S + dt B x^T; y = S^T C + D[h] x
+ * xbc rows (in `dtype`): [x: heads * vdim | B: groups * state_size | C: groups * state_size]; y fp32 [T, heads * vdim].
+ * state_size, vdim <= 256.                                                                                           */
+SP_API int sp_mamba2_scan(float* y, int64_t y_stride, const void* xbc, int64_t xbc_stride, const float* dt_raw,
+                          const float* dt_bias, const float* A_log, const float* Dskip, float* state, int64_t state_stride,
+                          int heads, int groups, int state_size, int vdim, SP_SEQ_PARAMS, int dtype, void* stream);
+/* out = (y * silu(z)) / rms_part * weight: each row of n values normed in `parts` equal parts (y fp32; z, out in `dtype`) */
+SP_API int sp_gated_group_norm(void* out, int64_t out_stride, const float* y, int64_t y_stride, const void* z,
+                               int64_t z_stride, const float* weight, int64_t num_tokens, int n, int parts, float eps,
+                               int dtype, void* stream);
+/* Per (request, head) over the request's rows in order, state (S [dim, vdim], n [dim], m) fp32, zero for a new sequence:
+ *   i = cap tanh(ipre / cap); f = logsigmoid(cap tanh(fpre / cap)); m' = max(f + m, i)
+ *   S = exp(f + m - m') S + exp(i - m') k v^T;  n likewise with k;  o = S^T q / (max(|n . q|, exp(-m')) + 1e-6), q scaled
+ *   by dim^(-1/2);  out = o / rms_head(o) * norm_w * sigmoid(g).   ipre, fpre fp32 [T, heads].  dim, vdim <= 256.    */
+SP_API int sp_mlstm_scan(void* out, int64_t out_stride, const void* q, int64_t q_stride, const void* k, int64_t k_stride,
+                         const void* v, int64_t v_stride, const void* g, int64_t g_stride, const float* ipre,
+                         const float* fpre, const float* norm_w, float* S_state, int64_t S_stride, float* n_state,
+                         int64_t n_stride, float* m_state, int64_t m_stride, int heads, int dim, int vdim, float cap,
+                         float eps, SP_SEQ_PARAMS, int dtype, void* stream);
 
 #ifdef __cplusplus
 }

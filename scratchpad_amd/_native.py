@@ -124,6 +124,23 @@ SIGNATURES = {
     "sp_moe_grouped_gemm": (_i32, [_vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _i64, _i64, _i32, _vp]),
     "sp_moe_glu": (_i32, [_vp, _vp, _i64, _i32, _f32, _f32, _i32, _vp]),
     "sp_moe_combine": (_i32, [_vp, _vp, _vp, _vp, _i64, _i32, _i32, _i64, _i32, _vp]),
+    # ---- ABI 11
+    "sp_moe_route_softmax": (_i32, [_vp, _vp, _vp, _i64, _vp, _i64, _i32, _i32, _i32, _f32, _i32, _vp]),
+    "sp_embed_scale": (_i32, [_vp, _i64, _vp, _vp, _i64, _i32, _i64, _f32, _i32, _vp]),
+    "sp_norm_shift": (_i32, [_vp, _vp, _i64, _vp, _i64, _vp, _vp, _vp, _i64, _i64, _i32, _f32, *_SEQ, _i32, _vp]),
+    "sp_norm_save_last": (_i32, [_vp, _i64, _vp, _i64, _vp, _i32, _f32, *_SEQ, _vp]),
+    "sp_stream_add": (_i32, [_vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _i64, _i32, _i32, _vp]),
+    "sp_qkv_rotary_store": (_i32, [_vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _vp, _f32, _i64, _i32,
+                                   _i32, _i32, _i32, _i32, _f32, _i32, _vp]),
+    "sp_pool_blocks": (_i32, [_vp, _vp, _vp, _vp, _i64, _i64, _vp, _i64, _i64, _i32, _i32, _i32, *_SEQ, _i32, _vp]),
+    "sp_window_attention": (_i32, [_vp, _i64, _vp, _i64, _vp, _vp, _vp, _vp, _i64, _i64, _vp, _i64, _i64, _i32, _i32, _i32,
+                                   _i32, _i64, _i32, _f32, *_SEQ, _i32, _vp]),
+    "sp_small_linear_f32": (_i32, [_vp, _vp, _i64, _vp, _vp, _i64, _i32, _i32, _i32, _vp]),
+    "sp_causal_conv_silu": (_i32, [_vp, _i64, _vp, _i64, _vp, _vp, _vp, _i64, _i64, _i32, _i32, *_SEQ, _i32, _vp]),
+    "sp_mamba2_scan": (_i32, [_vp, _i64, _vp, _i64, _vp, _vp, _vp, _vp, _vp, _i64, _i32, _i32, _i32, _i32, *_SEQ, _i32, _vp]),
+    "sp_gated_group_norm": (_i32, [_vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _i32, _i32, _f32, _i32, _vp]),
+    "sp_mlstm_scan": (_i32, [_vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _vp, _vp, _i64, _vp, _i64, _vp,
+                             _i64, _i32, _i32, _i32, _f32, _f32, *_SEQ, _i32, _vp]),
 }
 
 
@@ -157,7 +174,7 @@ def load() -> ctypes.CDLL:
             continue
         fn.restype = res
         fn.argtypes = args
-    if lib.sp_abi_version() != 10:
+    if lib.sp_abi_version() != 11:
         raise RuntimeError("libscratchpad_hip.so ABI version mismatch")
     _lib = lib
     return lib
@@ -1171,4 +1188,190 @@ def moe_combine(z: torch.Tensor, place: torch.Tensor, weights: torch.Tensor) -> 
     out = empty_rows(T, z.shape[1], z.dtype, z.device)
     _check(load().sp_moe_combine(out.data_ptr(), z.data_ptr(), place.data_ptr(), weights.data_ptr(), T, z.shape[1], top,
                                  out.stride(0), _dt(z), _stream()), "sp_moe_combine")
+    return out
+
+
+# --------------------------------------------------------------------------- fp32 stream with token shift, windowed attention, scans
+def moe_route_softmax(x: torch.Tensor, router: torch.Tensor, top: int, scale: float):
+    """(ids int32 [T, top], weights fp32 [T, top]): the largest softmax scores, times scale"""
+    _mat(x, "x"), _f32(router, "router")
+    T, E = x.shape[0], router.shape[0]
+    if router.shape[1] != x.shape[1]:
+        raise RuntimeError("moe_route_softmax: router [experts, width]")
+    ids = torch.empty((T, top), dtype=torch.int32, device=x.device)
+    weights = torch.empty((T, top), dtype=torch.float32, device=x.device)
+    _check(load().sp_moe_route_softmax(ids.data_ptr(), weights.data_ptr(), x.data_ptr(), x.stride(0), router.data_ptr(), T,
+                                       x.shape[1], E, top, scale, _dt(x), _stream()), "sp_moe_route_softmax")
+    return ids, weights
+
+
+def embed_scale(embed: torch.Tensor, ids: torch.Tensor, scale: float) -> torch.Tensor:
+    """fp32 [T, W] = embed[ids] * scale"""
+    _gpu(embed, ids)
+    if ids.dtype != torch.int64 or embed.dim() != 2 or not embed.is_contiguous():
+        raise RuntimeError("embed_scale: int64 ids, contiguous table [vocab, width]")
+    x = torch.empty((ids.shape[0], embed.shape[1]), dtype=torch.float32, device=embed.device)
+    _check(load().sp_embed_scale(x.data_ptr(), x.stride(0), embed.data_ptr(), ids.data_ptr(), ids.shape[0], embed.shape[1],
+                                 embed.shape[0], scale, _dt(embed), _stream()), "sp_embed_scale")
+    return x
+
+
+def norm_shift(x: torch.Tensor, weight: torch.Tensor, eps: float, dtype: torch.dtype, mu: Optional[torch.Tensor] = None,
+               state: Optional[torch.Tensor] = None, seq: Optional[SeqParams] = None, want_h: bool = True):
+    """(h, hs) in dtype: h = x / rms(x) * weight, hs = h + (h[t-1] - h) * mu (None without mu).  With mu, the request's
+    saved h (``state`` [slots, W] fp32) precedes a step's first row and is replaced by the step's last h."""
+    _mat(x, "x"), _f32(weight, "weight")
+    if x.dtype != torch.float32 or weight.shape[0] != x.shape[1]:
+        raise RuntimeError("norm_shift: x fp32 [T, W], weight [W]")
+    T, W = x.shape
+    h = empty_rows(T, W, dtype, x.device) if want_h or mu is None else None
+    hs = None
+    if mu is not None:
+        _f32(mu, "mu"), _f32(state, "state")
+        if seq is None or seq.num_tokens != T or state.shape[1] != W or mu.shape[0] != W:
+            raise RuntimeError("norm_shift: mu [W], state [slots, W] and the step's SeqParams go together")
+        hs = empty_rows(T, W, dtype, x.device)
+    stride = (h if h is not None else hs).stride(0)
+    args = seq.args if seq is not None else [None] * 6 + [0, 0]
+    _check(load().sp_norm_shift(_ptr(h), _ptr(hs), stride, x.data_ptr(), x.stride(0), weight.data_ptr(), _ptr(mu), _ptr(state),
+                                0 if state is None else state.stride(0), T, W, eps, *args, _DTYPES[dtype], _stream()),
+           "sp_norm_shift")
+    if mu is not None:
+        _check(load().sp_norm_save_last(state.data_ptr(), state.stride(0), x.data_ptr(), x.stride(0), weight.data_ptr(), W, eps,
+                                        *seq.args, _stream()), "sp_norm_save_last")
+    return h, hs
+
+
+def stream_add(x: torch.Tensor, a: torch.Tensor, b: Optional[torch.Tensor] = None, c: Optional[torch.Tensor] = None) -> None:
+    """x += a + b + c in place (x fp32)"""
+    _mat(x, "x")
+    if x.dtype != torch.float32:
+        raise RuntimeError("stream_add: x must be fp32")
+    for t in (a, b, c):
+        if t is not None and (_mat(t, "addend").shape != x.shape or t.dtype != a.dtype):
+            raise RuntimeError("stream_add: addends [T, W] of one dtype")
+    _check(load().sp_stream_add(x.data_ptr(), x.stride(0), a.data_ptr(), a.stride(0), _ptr(b), 0 if b is None else b.stride(0),
+                                _ptr(c), 0 if c is None else c.stride(0), x.shape[0], x.shape[1], _dt(a), _stream()),
+           "sp_stream_add")
+
+
+def qkv_rotary_store(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, kpool: torch.Tensor, vpool: torch.Tensor,
+                     positions: torch.Tensor, loc: torch.Tensor, freq: Optional[torch.Tensor], mag: float, heads: int,
+                     kv_heads: int, dim: int, vdim: int, eps: float) -> None:
+    """q [T, heads * dim] rotated in place; k rotated, v head-normed into the pools' rows loc (views: strides are taken)"""
+    for name, t, n in (("q", q, heads * dim), ("k", k, kv_heads * dim), ("v", v, kv_heads * vdim)):
+        if _mat(t, name).shape[1] != n or t.dtype != q.dtype or t.shape[0] != q.shape[0]:
+            raise RuntimeError(f"qkv_rotary_store: {name} must be [T, {n}]")
+    if kpool.dtype != q.dtype or vpool.dtype != q.dtype or _mat(kpool, "kpool").shape[1] != kv_heads * dim or \
+            _mat(vpool, "vpool").shape[1] != kv_heads * vdim:
+        raise RuntimeError("qkv_rotary_store: pools [P, kv_heads * dim] / [P, kv_heads * vdim] of q's dtype")
+    if positions.dtype != torch.int64 or loc.dtype != torch.int64 or loc.shape[0] != q.shape[0] or positions.shape[0] != q.shape[0]:
+        raise RuntimeError("qkv_rotary_store: int64 positions and loc, one per row")
+    dims = 0 if freq is None else 2 * _f32(freq, "freq").shape[0]
+    _check(load().sp_qkv_rotary_store(q.data_ptr(), q.stride(0), k.data_ptr(), k.stride(0), v.data_ptr(), v.stride(0),
+                                      kpool.data_ptr(), kpool.stride(0), vpool.data_ptr(), vpool.stride(0), positions.data_ptr(),
+                                      loc.data_ptr(), _ptr(freq), mag, q.shape[0], heads, kv_heads, dim, vdim, dims, eps, _dt(q),
+                                      _stream()), "sp_qkv_rotary_store")
+
+
+def pool_blocks(kpooled: torch.Tensor, vpooled: torch.Tensor, kpool: torch.Tensor, vpool: torch.Tensor,
+                req_to_token: torch.Tensor, seq: SeqParams, block: int) -> None:
+    if kpooled.shape != kpool.shape or vpooled.shape != vpool.shape or kpooled.dtype != kpool.dtype or \
+            kpooled.stride(0) != kpool.stride(0) or vpooled.stride(0) != vpool.stride(0) or req_to_token.dtype != torch.int32:
+        raise RuntimeError("pool_blocks: pooled buffers must mirror the token buffers")
+    _check(load().sp_pool_blocks(kpooled.data_ptr(), vpooled.data_ptr(), kpool.data_ptr(), vpool.data_ptr(), kpool.stride(0),
+                                 vpool.stride(0), req_to_token.data_ptr(), req_to_token.stride(0), seq.num_tokens,
+                                 kpool.shape[1], vpool.shape[1], block, *seq.args, _dt(kpool), _stream()), "sp_pool_blocks")
+
+
+def window_attention(q: torch.Tensor, kpool: torch.Tensor, vpool: torch.Tensor, kpooled: Optional[torch.Tensor],
+                     vpooled: Optional[torch.Tensor], req_to_token: torch.Tensor, seq: SeqParams, heads: int, kv_heads: int,
+                     dim: int, vdim: int, window: int, block: int, scale: float) -> torch.Tensor:
+    """q [T, heads * dim] (rotated) -> [T, heads * vdim]"""
+    _mat(q, "q"), _mat(kpool, "kpool"), _mat(vpool, "vpool")
+    T = q.shape[0]
+    if q.shape[1] != heads * dim or kpool.shape[1] != kv_heads * dim or vpool.shape[1] != kv_heads * vdim or \
+            kpool.dtype != q.dtype or vpool.dtype != q.dtype or req_to_token.dtype != torch.int32 or T != seq.num_tokens:
+        raise RuntimeError("window_attention: shapes / dtypes do not fit")
+    if kpooled is not None and (kpooled.stride(0) != kpool.stride(0) or vpooled.stride(0) != vpool.stride(0)):
+        raise RuntimeError("window_attention: pooled buffers must mirror the token buffers")
+    out = empty_rows(T, heads * vdim, q.dtype, q.device)
+    _check(load().sp_window_attention(out.data_ptr(), out.stride(0), q.data_ptr(), q.stride(0), kpool.data_ptr(),
+                                      vpool.data_ptr(), _ptr(kpooled), _ptr(vpooled), kpool.stride(0), vpool.stride(0),
+                                      req_to_token.data_ptr(), req_to_token.stride(0), T, heads, kv_heads, dim, vdim,
+                                      window, block, scale, *seq.args, _dt(q), _stream()), "sp_window_attention")
+    return out
+
+
+def small_linear_f32(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """fp32 [T, n] = x @ weight.T + bias with fp32 weights, accumulation and output (gates and step sizes of recurrences)"""
+    _mat(x, "x"), _f32(weight, "weight")
+    if weight.dim() != 2 or weight.shape[1] != x.shape[1] or (bias is not None and _f32(bias, "bias").shape[0] != weight.shape[0]):
+        raise RuntimeError("small_linear_f32: weight [n, k], bias [n]")
+    out = torch.empty((x.shape[0], weight.shape[0]), dtype=torch.float32, device=x.device)
+    _check(load().sp_small_linear_f32(out.data_ptr(), x.data_ptr(), x.stride(0), weight.data_ptr(), _ptr(bias), x.shape[0],
+                                      x.shape[1], weight.shape[0], _dt(x), _stream()), "sp_small_linear_f32")
+    return out
+
+
+def causal_conv_silu(u: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], state: torch.Tensor,
+                     seq: SeqParams) -> torch.Tensor:
+    """u [T, C] (a view: its row stride is taken) -> silu(conv) [T, C]; state [slots, taps - 1, C] fp32 is read and moved on"""
+    _mat(u, "u"), _f32(weight, "weight"), _f32(state, "state")
+    C, taps = weight.shape
+    if u.shape[1] != C or u.shape[0] != seq.num_tokens or state.shape[1:] != (max(taps - 1, 0), C) or \
+            (bias is not None and _f32(bias, "bias").shape[0] != C):
+        raise RuntimeError("causal_conv_silu: u [num_tokens, C], weight [C, taps], state [slots, taps - 1, C]")
+    out = empty_rows(u.shape[0], C, u.dtype, u.device)
+    _check(load().sp_causal_conv_silu(out.data_ptr(), out.stride(0), u.data_ptr(), u.stride(0), weight.data_ptr(), _ptr(bias),
+                                      state.data_ptr(), state.stride(0), u.shape[0], C, taps, *seq.args, _dt(u), _stream()),
+           "sp_causal_conv_silu")
+    return out
+
+
+def mamba2_scan(xbc: torch.Tensor, dt_raw: torch.Tensor, dt_bias: torch.Tensor, A_log: torch.Tensor, D: torch.Tensor,
+                state: torch.Tensor, seq: SeqParams, heads: int, groups: int, state_size: int, vdim: int) -> torch.Tensor:
+    """xbc [T, heads * vdim + 2 * groups * state_size] -> y fp32 [T, heads * vdim]; state [slots, heads, state_size, vdim]"""
+    _mat(xbc, "xbc"), _f32(dt_raw, "dt_raw"), _f32(dt_bias, "dt_bias"), _f32(A_log, "A_log"), _f32(D, "D"), _f32(state, "state")
+    inner = heads * vdim
+    if xbc.shape != (seq.num_tokens, inner + 2 * groups * state_size) or dt_raw.shape != (seq.num_tokens, heads) or \
+            state.shape[1:] != (heads, state_size, vdim) or dt_bias.numel() != heads or A_log.numel() != heads or D.numel() != heads:
+        raise RuntimeError("mamba2_scan: shapes do not fit")
+    y = torch.empty((xbc.shape[0], inner), dtype=torch.float32, device=xbc.device)
+    _check(load().sp_mamba2_scan(y.data_ptr(), y.stride(0), xbc.data_ptr(), xbc.stride(0), dt_raw.data_ptr(), dt_bias.data_ptr(),
+                                 A_log.data_ptr(), D.data_ptr(), state.data_ptr(), state.stride(0), heads, groups, state_size,
+                                 vdim, *seq.args, _dt(xbc), _stream()), "sp_mamba2_scan")
+    return y
+
+
+def gated_group_norm(y: torch.Tensor, z: torch.Tensor, weight: torch.Tensor, parts: int, eps: float) -> torch.Tensor:
+    """(y * silu(z)) normed in `parts` equal parts, times weight; y fp32, z (a view) and the result in z's dtype"""
+    _mat(y, "y"), _mat(z, "z"), _f32(weight, "weight")
+    if y.dtype != torch.float32 or y.shape != z.shape or weight.shape[0] != y.shape[1] or y.shape[1] % parts:
+        raise RuntimeError("gated_group_norm: y fp32 [T, n], z [T, n], weight [n], n divisible by parts")
+    out = empty_rows(y.shape[0], y.shape[1], z.dtype, y.device)
+    _check(load().sp_gated_group_norm(out.data_ptr(), out.stride(0), y.data_ptr(), y.stride(0), z.data_ptr(), z.stride(0),
+                                      weight.data_ptr(), y.shape[0], y.shape[1], parts, eps, _dt(z), _stream()),
+           "sp_gated_group_norm")
+    return out
+
+
+def mlstm_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, g: torch.Tensor, ipre: torch.Tensor, fpre: torch.Tensor,
+               norm_w: torch.Tensor, S: torch.Tensor, n: torch.Tensor, m: torch.Tensor, seq: SeqParams, heads: int, dim: int,
+               vdim: int, cap: float, eps: float) -> torch.Tensor:
+    """q, k [T, heads * dim], v, g [T, heads * vdim] (views) -> [T, heads * vdim]; states S [slots, heads, dim, vdim],
+    n [slots, heads, dim], m [slots, heads] fp32"""
+    T = seq.num_tokens
+    for name, t, w in (("q", q, heads * dim), ("k", k, heads * dim), ("v", v, heads * vdim), ("g", g, heads * vdim)):
+        if _mat(t, name).shape != (T, w) or t.dtype != q.dtype:
+            raise RuntimeError(f"mlstm_scan: {name} must be [num_tokens, {w}] of one dtype")
+    _f32(ipre, "ipre"), _f32(fpre, "fpre"), _f32(norm_w, "norm_w"), _f32(S, "S"), _f32(n, "n"), _f32(m, "m")
+    if ipre.shape != (T, heads) or fpre.shape != (T, heads) or norm_w.numel() != heads * vdim or \
+            S.shape[1:] != (heads, dim, vdim) or n.shape[1:] != (heads, dim) or m.shape[1:] != (heads,):
+        raise RuntimeError("mlstm_scan: gate or state shapes do not fit")
+    out = empty_rows(T, heads * vdim, q.dtype, q.device)
+    _check(load().sp_mlstm_scan(out.data_ptr(), out.stride(0), q.data_ptr(), q.stride(0), k.data_ptr(), k.stride(0),
+                                v.data_ptr(), v.stride(0), g.data_ptr(), g.stride(0), ipre.data_ptr(), fpre.data_ptr(),
+                                norm_w.data_ptr(), S.data_ptr(), S.stride(0), n.data_ptr(), n.stride(0), m.data_ptr(),
+                                m.stride(0), heads, dim, vdim, cap, eps, *seq.args, _dt(q), _stream()), "sp_mlstm_scan")
     return out

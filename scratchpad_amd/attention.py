@@ -533,9 +533,34 @@ class LatentAttention(nn.Module):
         return forward_batch.attn_backend.forward_latent(q_lat, q_rot, self, forward_batch)
 
 
+class PooledWindowAttention(nn.Module):
+    """Layer-local constants of a grouped-query attention layer over a WindowKVPool: a query sees the ``window`` latest
+    tokens and, for every block of ``block`` positions wholly behind the window, the block's mean key and value (one
+    softmax over both); key width ``dim`` and value width ``vdim`` may differ.  window None: plain causal attention."""
+
+    def __init__(self, num_heads: int, num_kv_heads: int, dim: int, vdim: int, scaling: float, layer_id: int,
+                 window: Optional[int] = None, block: Optional[int] = None):
+        super().__init__()
+        if num_heads % num_kv_heads:
+            raise ValueError("query heads must be a multiple of key/value heads")
+        self.tp_q_head_num, self.tp_k_head_num = num_heads, num_kv_heads
+        self.dim, self.vdim, self.scaling, self.layer_id = dim, vdim, scaling, layer_id
+        self.window = int(window) if window else 0
+        self.block = int(block) if (block and window) else 0
+
+    def store(self, q, k, v, rotary, positions, eps: float, forward_batch: "ForwardBatch") -> None:
+        """rotate q in place; rotate k, norm v per head and put both into the pool; then the blocks this step completes"""
+        forward_batch.attn_backend.store_window(q, k, v, rotary, positions, eps, self, forward_batch)
+
+    def forward(self, q, forward_batch: "ForwardBatch"):
+        """q [T, heads * dim] (rotated) -> [T, heads * vdim]; the step's rows are in the pool"""
+        return forward_batch.attn_backend.forward_window(q, self, forward_batch)
+
+
 class SequenceBackend(AttentionBackend):
     """Backend of models whose layers read per-request state through the step's request table instead of a planned
-    key/value gather: latent attention layers (LatentTokenToKVPool) and recurrent layers (RecurrentStatePool).  Its
+    key/value gather: latent attention layers (LatentTokenToKVPool), windowed attention layers with pooled blocks
+    (WindowKVPool) and recurrent layers (RecurrentStatePool).  Its
     per-step metadata is the kernels' request description (_native.SeqParams), built once per forward; launches read
     req_pool_indices / seq_lens from the batch's own tensors, so a captured decode step replays on the graph runner's
     static buffers with nothing to rebuild."""
@@ -574,7 +599,25 @@ class SequenceBackend(AttentionBackend):
         return _native.latent_attention(q_lat, q_rot, pool, forward_batch.req_to_token_pool.req_to_token, self.seq,
                                         layer.scaling)
 
+    def store_window(self, q, k, v, rotary, positions, eps, layer: "PooledWindowAttention", forward_batch: "ForwardBatch"):
+        pool = forward_batch.token_to_kv_pool
+        kbuf, vbuf = pool.get_kv_buffer(layer.layer_id)
+        freq, mag = (rotary.freq, rotary.magnitude) if rotary is not None else (None, 1.0)
+        _native.qkv_rotary_store(q, k, v, kbuf, vbuf, positions, forward_batch.out_cache_loc, freq, mag, layer.tp_q_head_num,
+                                 layer.tp_k_head_num, layer.dim, layer.vdim, eps)
+        if layer.block:
+            kp, vp = pool.get_pooled_buffers(layer.layer_id)
+            _native.pool_blocks(kp, vp, kbuf, vbuf, forward_batch.req_to_token_pool.req_to_token, self.seq, layer.block)
+
+    def forward_window(self, q, layer: "PooledWindowAttention", forward_batch: "ForwardBatch"):
+        pool = forward_batch.token_to_kv_pool
+        kbuf, vbuf = pool.get_kv_buffer(layer.layer_id)
+        kp, vp = pool.get_pooled_buffers(layer.layer_id) if layer.block else (None, None)
+        return _native.window_attention(q, kbuf, vbuf, kp, vp, forward_batch.req_to_token_pool.req_to_token, self.seq,
+                                        layer.tp_q_head_num, layer.tp_k_head_num, layer.dim, layer.vdim, layer.window,
+                                        layer.block, layer.scaling)
+
     def forward_decode(self, q, k, v, layer, forward_batch, save_kv_cache: bool = True):
-        raise NotImplementedError("this backend serves latent attention layers (forward_latent)")
+        raise NotImplementedError("this backend serves latent attention layers (forward_latent) and windowed ones (forward_window)")
 
     forward_extend = forward_decode

@@ -79,6 +79,59 @@ __global__ void moe_route_kernel(int32_t* ids, float* weights, const void* x, in
   }
 }
 
+// ---- router with softmax scores: one wave per token -----------------------------------------------------------------
+// z = W x (fp32), s = softmax(z) over all experts; the `top` largest s win (ties: the lower index); weights = s * scale
+template <typename Tag>
+__global__ void moe_route_softmax_kernel(int32_t* ids, float* weights, const void* x, int64_t x_stride, const float* router,
+                                         int64_t T, int width, int E, int top, float scale) {
+  typedef Elem<Tag> El;
+  extern __shared__ float smem[];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int64_t t = (int64_t)blockIdx.x * (blockDim.x >> 6) + wave;
+  if (t >= T) return;
+  float* score = smem + (size_t)wave * 2 * E;     // s[E], then the choice copy
+  float* choice = score + E;
+  float zmax = -INFINITY;
+  for (int e = 0; e < E; ++e) {
+    float d = 0.f;
+    for (int i = lane; i < width; i += 64) d += router[(int64_t)e * width + i] * El::load(x, t * x_stride + i);
+    d = wave_sum(d);
+    zmax = fmaxf(zmax, d);
+    if (lane == 0) score[e] = d;
+  }
+  __builtin_amdgcn_wave_barrier();
+  float part = 0.f;
+  for (int e = lane; e < E; e += 64) part += expf(score[e] - zmax);
+  const float inv = 1.f / wave_sum(part);
+  for (int e = lane; e < E; e += 64) {
+    const float sv = expf(score[e] - zmax) * inv;
+    score[e] = sv;
+    choice[e] = sv;
+  }
+  __builtin_amdgcn_wave_barrier();
+  for (int k = 0; k < top; ++k) {
+    float best = -INFINITY;
+    int at = 0x7fffffff;
+    for (int e = lane; e < E; e += 64) {
+      const float c = choice[e];
+      if (c > best) { best = c; at = e; }
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+      const float ob = __shfl_xor(best, off, 64);
+      const int oa = __shfl_xor(at, off, 64);
+      if (ob > best || (ob == best && oa < at)) { best = ob; at = oa; }
+    }
+    if (at >= E) at = 0;
+    if (lane == 0) {
+      ids[t * top + k] = at;
+      weights[t * top + k] = score[at] * scale;
+      choice[at] = -INFINITY;
+    }
+    __builtin_amdgcn_wave_barrier();
+  }
+}
+
 // ---- pairs ordered by expert: offsets[E + 1], order[pos] = pair, place[pair] = pos.  One workgroup. ---------------
 __global__ void moe_align_kernel(int32_t* offsets, int32_t* order, int32_t* place, const int32_t* ids, int P, int E) {
   extern __shared__ int32_t cnt[];          // counts[E], then cursors[E]
@@ -308,6 +361,20 @@ extern "C" int sp_moe_route(int32_t* ids, float* weights, const void* x, int64_t
   if (lds > 64 * 1024) return SP_ERR_UNSUPPORTED;
   SP_DISPATCH_DTYPE(dtype, (moe_route_kernel<Tag><<<dim3((unsigned)((num_tokens + 3) / 4)), 256, lds, (hipStream_t)stream>>>(
                                ids, weights, x, x_stride, router, correction, num_tokens, width, experts, top, groups, keep)));
+  SP_LAUNCH_CHECK();
+  return SP_OK;
+}
+
+extern "C" int sp_moe_route_softmax(int32_t* ids, float* weights, const void* x, int64_t x_stride, const float* router,
+                                    int64_t num_tokens, int width, int experts, int top, float scale, int dtype,
+                                    void* stream) {
+  SP_CHECK_ARG(num_tokens >= 0 && width > 0 && experts > 0 && top > 0 && top <= experts);
+  if (num_tokens == 0) return SP_OK;
+  SP_CHECK_ARG(ids && weights && x && router && x_stride >= width);
+  const size_t lds = 4 * (size_t)(2 * experts) * sizeof(float);
+  if (lds > 64 * 1024) return SP_ERR_UNSUPPORTED;
+  SP_DISPATCH_DTYPE(dtype, (moe_route_softmax_kernel<Tag><<<dim3((unsigned)((num_tokens + 3) / 4)), 256, lds, (hipStream_t)stream>>>(
+                               ids, weights, x, x_stride, router, num_tokens, width, experts, top, scale)));
   SP_LAUNCH_CHECK();
   return SP_OK;
 }

@@ -1,0 +1,255 @@
+// State-space mixer (Mamba-2 form) and the small pieces recurrent mixers share.
+//   gate projections   out[t, n] = bias[n] + sum_i w[n, i] x[t, i]        few outputs (one per head), fp32 weights,
+//                                                                         fp32 accumulation and fp32 OUTPUT: what enters
+//                                                                         a recurrence's decay or gate is never rounded
+//   causal convolution out[t, c] = silu(bias[c] + sum_j w[c, j] in[t - (taps-1) + j, c])   per channel; inputs before a
+//                      step's first row come from the request's saved last taps-1 inputs (zeros before the sequence)
+//   scan               dt = softplus(dt_raw + dt_bias);  S <- exp(-exp(A_log) dt) S + dt B x^T;  y = S^T C + D x
+//                      per head, S [N, Dv] fp32 in the state pool; head h reads B, C of group h / (H / G)
+//   gated group norm   out = (y silu(z)) / rms_part * w      the gate BEFORE the norm, `parts` equal parts per row
+#include "seq_batch.h"
+
+namespace sp {
+namespace {
+
+__device__ __forceinline__ float softplus_f(float z) { return fmaxf(z, 0.f) + log1pf(expf(-fabsf(z))); }
+
+// one wave per token, all outputs in turn
+template <typename Tag>
+__global__ void __launch_bounds__(256)
+small_linear_f32_kernel(float* out, const void* x, int64_t x_stride, const float* w, const float* bias, int64_t T, int K, int N) {
+  typedef Elem<Tag> E;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int64_t t = (int64_t)blockIdx.x * 4 + wave;
+  if (t >= T) return;
+  for (int n = 0; n < N; ++n) {
+    float d = 0.f;
+    for (int i = lane; i < K; i += 64) d += w[(int64_t)n * K + i] * E::load(x, t * x_stride + i);
+    d = wave_sum(d);
+    if (lane == 0) out[t * N + n] = d + (bias ? bias[n] : 0.f);
+  }
+}
+
+// state [slot][taps - 1][C]: entry k = the input at position (tokens held) - (taps - 1) + k
+template <typename Tag>
+__global__ void __launch_bounds__(kBlock)
+conv_silu_kernel(void* out, int64_t out_stride, const void* in, int64_t in_stride, const float* w, const float* bias,
+                 const float* state, int64_t state_stride, SeqBatch s, int C, int taps) {
+  typedef Elem<Tag> E;
+  const int64_t t = blockIdx.x;
+  const int c = blockIdx.y * kBlock + threadIdx.x;
+  if (c >= C) return;
+  int b;
+  int64_t start, prefix;
+  seq_of_token(s, t, b, start, prefix);
+  const float* st = state + load_idx(s.req_pool_indices, b, s.idx64) * state_stride;
+  float acc = bias ? bias[c] : 0.f;
+  for (int j = 0; j < taps; ++j) {
+    const int64_t r = t - (taps - 1) + j;
+    float val = 0.f;
+    if (r >= start) {
+      val = E::load(in, r * in_stride + c);
+    } else {
+      const int64_t back = start - r;                  // 1 .. taps - 1 rows before the step
+      if (prefix - back >= 0) val = st[(int64_t)(taps - 1 - back) * C + c];
+    }
+    acc += w[(int64_t)c * taps + j] * val;
+  }
+  E::store(out, t * out_stride + c, acc / (1.f + expf(-acc)));
+}
+
+constexpr int kMaxTaps = 16;
+
+template <typename Tag>
+__global__ void __launch_bounds__(kBlock)
+conv_state_kernel(float* state, int64_t state_stride, const void* in, int64_t in_stride, SeqBatch s, int C, int taps) {
+  typedef Elem<Tag> E;
+  const int b = blockIdx.x;
+  const int c = blockIdx.y * kBlock + threadIdx.x;
+  if (c >= C) return;
+  int64_t start, len, prefix;
+  seq_span(s, b, start, len, prefix);
+  if (len <= 0) return;
+  float* st = state + load_idx(s.req_pool_indices, b, s.idx64) * state_stride;
+  const int keep = taps - 1;
+  float fresh[kMaxTaps];
+  for (int k = 0; k < keep; ++k) {
+    const int64_t p = prefix + len - keep + k;       // position of the new entry k
+    float val = 0.f;
+    if (p >= prefix) val = E::load(in, (start + (p - prefix)) * in_stride + c);
+    else if (p >= 0) val = st[(p - prefix + keep) * C + c];
+    fresh[k] = val;
+  }
+  for (int k = 0; k < keep; ++k) st[(int64_t)k * C + c] = fresh[k];
+}
+
+constexpr int kChunk = 8;       // tokens staged in LDS per pass
+
+// one workgroup per (request, head); thread j owns column j of S (N values in registers)
+template <typename Tag, int NP>
+__global__ void __launch_bounds__(256)
+mamba2_scan_kernel(float* y, int64_t y_stride, const void* xbc, int64_t xbc_stride, const float* dt_raw, const float* dt_bias,
+                   const float* A_log, const float* Dskip, float* state, int64_t state_stride, SeqBatch s, int H, int G, int N,
+                   int Dv) {
+  typedef Elem<Tag> E;
+  __shared__ float sB[kChunk][NP], sC[kChunk][NP], sdt[kChunk], sdec[kChunk];
+  const int b = blockIdx.x, h = blockIdx.y, j = threadIdx.x;
+  const int nthreads = blockDim.x;
+  int64_t start, len, prefix;
+  seq_span(s, b, start, len, prefix);
+  if (len <= 0) return;
+  const bool live = j < Dv;
+  const int g = h / (H / G);
+  const int64_t inner = (int64_t)H * Dv;
+  const int64_t colx = (int64_t)h * Dv, colB = inner + (int64_t)g * N, colC = inner + (int64_t)G * N + (int64_t)g * N;
+  float* st = state + load_idx(s.req_pool_indices, b, s.idx64) * state_stride + (int64_t)h * N * Dv;
+  float S[NP];
+#pragma unroll
+  for (int i = 0; i < NP; ++i) S[i] = (live && i < N && prefix > 0) ? st[(int64_t)i * Dv + j] : 0.f;
+  const float a = expf(A_log[h]), bias = dt_bias[h], skip = Dskip[h];
+  for (int64_t c0 = 0; c0 < len; c0 += kChunk) {
+    const int n = (int)(len - c0 < kChunk ? len - c0 : kChunk);
+    __syncthreads();
+    for (int e = j; e < n * NP; e += nthreads) {
+      const int tt = e / NP, i = e % NP;
+      const int64_t row = start + c0 + tt;
+      const bool ok = i < N;
+      sB[tt][i] = ok ? E::load(xbc, row * xbc_stride + colB + i) : 0.f;
+      sC[tt][i] = ok ? E::load(xbc, row * xbc_stride + colC + i) : 0.f;
+    }
+    if (j < n) {
+      const float dt = softplus_f(dt_raw[(start + c0 + j) * H + h] + bias);
+      sdt[j] = dt;
+      sdec[j] = expf(-a * dt);
+    }
+    __syncthreads();
+    for (int tt = 0; tt < n; ++tt) {
+      const int64_t row = start + c0 + tt;
+      const float xj = live ? E::load(xbc, row * xbc_stride + colx + j) : 0.f;
+      const float dec = sdec[tt], dx = sdt[tt] * xj;
+      float o = 0.f;
+#pragma unroll
+      for (int i = 0; i < NP; ++i) {
+        S[i] = dec * S[i] + sB[tt][i] * dx;
+        o += S[i] * sC[tt][i];
+      }
+      if (live) y[row * y_stride + colx + j] = o + skip * xj;
+    }
+  }
+  if (live) {
+#pragma unroll
+    for (int i = 0; i < NP; ++i)
+      if (i < N) st[(int64_t)i * Dv + j] = S[i];
+  }
+}
+
+template <typename Tag>
+__global__ void __launch_bounds__(kBlock)
+gated_group_norm_kernel(void* out, int64_t out_stride, const float* y, int64_t y_stride, const void* z, int64_t z_stride,
+                        const float* w, int n, int parts, float eps) {
+  typedef Elem<Tag> E;
+  __shared__ float red[kBlock / 64];
+  const int64_t t = blockIdx.x;
+  const int per = n / parts;
+  for (int p = 0; p < parts; ++p) {
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < per; i += blockDim.x) {
+      const float zv = E::load(z, t * z_stride + p * per + i);
+      const float v = y[t * y_stride + p * per + i] * (zv / (1.f + expf(-zv)));
+      ss += v * v;
+    }
+    ss = block_sum(ss, red);
+    const float inv = 1.f / sqrtf(ss / (float)per + eps);
+    for (int i = threadIdx.x; i < per; i += blockDim.x) {
+      const int c = p * per + i;
+      const float zv = E::load(z, t * z_stride + c);
+      E::store(out, t * out_stride + c, y[t * y_stride + c] * (zv / (1.f + expf(-zv))) * inv * w[c]);
+    }
+  }
+}
+
+}  // namespace
+}  // namespace sp
+
+using namespace sp;
+
+extern "C" int sp_small_linear_f32(float* out, const void* x, int64_t x_stride, const float* weight, const float* bias,
+                                   int64_t num_tokens, int k, int n, int dtype, void* stream) {
+  SP_CHECK_ARG(num_tokens >= 0 && k > 0 && n > 0);
+  if (num_tokens == 0) return SP_OK;
+  SP_CHECK_ARG(out && x && weight && x_stride >= k);
+  SP_DISPATCH_DTYPE(dtype, (small_linear_f32_kernel<Tag><<<dim3((unsigned)((num_tokens + 3) / 4)), 256, 0, (hipStream_t)stream>>>(
+                               out, x, x_stride, weight, bias, num_tokens, k, n)));
+  SP_LAUNCH_CHECK();
+  return SP_OK;
+}
+
+extern "C" int sp_causal_conv_silu(void* out, int64_t out_stride, const void* in, int64_t in_stride, const float* weight,
+                                   const float* bias, float* state, int64_t state_stride, int64_t num_tokens, int channels,
+                                   int taps, SP_SEQ_PARAMS, int dtype, void* stream) {
+  SP_CHECK_ARG(num_tokens >= 0 && channels > 0 && taps >= 1 && taps <= kMaxTaps);
+  if (num_tokens == 0) return SP_OK;
+  SP_CHECK_ARG(out && in && weight && state && req_pool_indices && seq_lens);
+  SP_CHECK_ARG(out_stride >= channels && in_stride >= channels && state_stride >= (int64_t)(taps - 1) * channels);
+  SP_CHECK_ARG(!extend_seq_lens || (extend_prefix_lens && extend_start_loc && token_req));
+  SP_CHECK_ARG(extend_seq_lens || num_tokens == batch_size);
+  SEQ_BATCH(s);
+  const unsigned cb = (unsigned)((channels + kBlock - 1) / kBlock);
+  SP_DISPATCH_DTYPE(dtype, (conv_silu_kernel<Tag><<<dim3((unsigned)num_tokens, cb), kBlock, 0, (hipStream_t)stream>>>(
+                               out, out_stride, in, in_stride, weight, bias, state, state_stride, s, channels, taps)));
+  SP_LAUNCH_CHECK();
+  if (taps > 1) {      // after every reader of the old state (stream order)
+    SP_DISPATCH_DTYPE(dtype, (conv_state_kernel<Tag><<<dim3((unsigned)batch_size, cb), kBlock, 0, (hipStream_t)stream>>>(
+                                 state, state_stride, in, in_stride, s, channels, taps)));
+    SP_LAUNCH_CHECK();
+  }
+  return SP_OK;
+}
+
+template <typename Tag>
+static int launch_mamba2(float* y, int64_t y_stride, const void* xbc, int64_t xbc_stride, const float* dt_raw,
+                         const float* dt_bias, const float* A_log, const float* Dskip, float* state, int64_t state_stride,
+                         const SeqBatch& s, int H, int G, int N, int Dv, hipStream_t st) {
+  const dim3 grid((unsigned)s.B, (unsigned)H);
+  const unsigned threads = (unsigned)((Dv + 63) / 64 * 64);
+#define SP_SCAN(NP)                                                                                                    \
+  mamba2_scan_kernel<Tag, NP><<<grid, threads, 0, st>>>(y, y_stride, xbc, xbc_stride, dt_raw, dt_bias, A_log, Dskip, state, \
+                                                        state_stride, s, H, G, N, Dv)
+  if (N <= 16) SP_SCAN(16);
+  else if (N <= 32) SP_SCAN(32);
+  else if (N <= 64) SP_SCAN(64);
+  else if (N <= 128) SP_SCAN(128);
+  else if (N <= 256) SP_SCAN(256);
+  else return SP_ERR_UNSUPPORTED;
+#undef SP_SCAN
+  SP_LAUNCH_CHECK();
+  return SP_OK;
+}
+
+extern "C" int sp_mamba2_scan(float* y, int64_t y_stride, const void* xbc, int64_t xbc_stride, const float* dt_raw,
+                              const float* dt_bias, const float* A_log, const float* Dskip, float* state,
+                              int64_t state_stride, int heads, int groups, int state_size, int vdim, SP_SEQ_PARAMS,
+                              int dtype, void* stream) {
+  SP_CHECK_ARG(batch_size >= 0 && heads > 0 && groups > 0 && heads % groups == 0 && state_size > 0 && vdim > 0 && vdim <= 256);
+  if (batch_size == 0) return SP_OK;
+  SP_CHECK_ARG(y && xbc && dt_raw && dt_bias && A_log && Dskip && state && req_pool_indices && seq_lens);
+  SP_CHECK_ARG(!extend_seq_lens || (extend_prefix_lens && extend_start_loc));
+  const int64_t inner = (int64_t)heads * vdim;
+  SP_CHECK_ARG(y_stride >= inner && xbc_stride >= inner + 2 * (int64_t)groups * state_size);
+  SP_CHECK_ARG(state_stride >= (int64_t)heads * state_size * vdim);
+  SEQ_BATCH(s);
+  SP_DISPATCH_DTYPE(dtype, return (launch_mamba2<Tag>(y, y_stride, xbc, xbc_stride, dt_raw, dt_bias, A_log, Dskip, state,
+                                                      state_stride, s, heads, groups, state_size, vdim, (hipStream_t)stream)));
+}
+
+extern "C" int sp_gated_group_norm(void* out, int64_t out_stride, const float* y, int64_t y_stride, const void* z,
+                                   int64_t z_stride, const float* weight, int64_t num_tokens, int n, int parts, float eps,
+                                   int dtype, void* stream) {
+  SP_CHECK_ARG(num_tokens >= 0 && n > 0 && parts > 0 && n % parts == 0);
+  if (num_tokens == 0) return SP_OK;
+  SP_CHECK_ARG(out && y && z && weight && out_stride >= n && y_stride >= n && z_stride >= n);
+  SP_DISPATCH_DTYPE(dtype, (gated_group_norm_kernel<Tag><<<dim3((unsigned)num_tokens), kBlock, 0, (hipStream_t)stream>>>(
+                               out, out_stride, y, y_stride, z, z_stride, weight, n, parts, eps)));
+  SP_LAUNCH_CHECK();
+  return SP_OK;
+}

@@ -1,0 +1,153 @@
+// fp32 residual stream of parallel-sublayer models:  x <- x + mixer(shift(h)) + ff(h),  h = x / rms(x) * w.
+//   scaled embedding      x[t]  = embed[id[t]] * scale                                     (fp32)
+//   norm + token shift    h[t]  = x[t] / sqrt(mean(x[t]^2) + eps) * w                      (what the feed-forward reads)
+//                         hs[t] = h[t] + (h[t-1] - h[t]) * mu                              (what the mixer reads)
+//                         h[-1] of a step's first row = the request's saved h (zeros at a sequence's first token)
+//   saved h               state[slot] = h[the request's last row of this step]             (fp32, a launch of its own:
+//                                                                                           every reader has finished)
+//   sum                   x[t] += a[t] + b[t] + c[t]                                       (fp32; b, c optional)
+// All arithmetic is fp32; h and hs are rounded once, to the projections' element type.
+#include "seq_batch.h"
+
+namespace sp {
+namespace {
+
+template <typename Tag>
+__global__ void embed_scale_kernel(float* x, int64_t x_stride, const void* embed, const int64_t* ids, int width,
+                                   int64_t vocab, float scale) {
+  typedef Elem<Tag> E;
+  const int64_t t = blockIdx.x;
+  int64_t id = ids[t];
+  id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);
+  for (int i = threadIdx.x; i < width; i += blockDim.x) x[t * x_stride + i] = E::load(embed, id * width + i) * scale;
+}
+
+// one workgroup per row: the row's own norm and, for the shift, the previous row's (recomputed: two reads of a row
+// are cheaper than a second launch and an fp32 copy of h)
+template <typename Tag>
+__global__ void __launch_bounds__(kBlock)
+norm_shift_kernel(void* out_h, void* out_hs, int64_t out_stride, const float* x, int64_t x_stride, const float* w,
+                  const float* mu, const float* state, int64_t state_stride, SeqBatch s, int width, float eps) {
+  typedef Elem<Tag> E;
+  __shared__ float red[kBlock / 64];
+  const int64_t t = blockIdx.x;
+  const float* row = x + t * x_stride;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < width; i += blockDim.x) ss += row[i] * row[i];
+  ss = block_sum(ss, red);
+  const float inv = 1.f / sqrtf(ss / (float)width + eps);
+  if (!out_hs) {
+    for (int i = threadIdx.x; i < width; i += blockDim.x) E::store(out_h, t * out_stride + i, row[i] * inv * w[i]);
+    return;
+  }
+  int b;
+  int64_t start, prefix;
+  seq_of_token(s, t, b, start, prefix);
+  const float* prow = nullptr;       // previous row of x (its norm is computed here)
+  const float* saved = nullptr;      // or the saved h
+  float pinv = 0.f;
+  if (t > start) {
+    prow = x + (t - 1) * x_stride;
+    float ps = 0.f;
+    for (int i = threadIdx.x; i < width; i += blockDim.x) ps += prow[i] * prow[i];
+    ps = block_sum(ps, red);
+    pinv = 1.f / sqrtf(ps / (float)width + eps);
+  } else if (prefix > 0) {
+    saved = state + load_idx(s.req_pool_indices, b, s.idx64) * state_stride;
+  }
+  for (int i = threadIdx.x; i < width; i += blockDim.x) {
+    const float h = row[i] * inv * w[i];
+    const float hp = prow ? prow[i] * pinv * w[i] : (saved ? saved[i] : 0.f);
+    if (out_h) E::store(out_h, t * out_stride + i, h);
+    E::store(out_hs, t * out_stride + i, h + (hp - h) * mu[i]);
+  }
+}
+
+// state[slot of request b] = h[last row of b]
+__global__ void __launch_bounds__(kBlock)
+norm_save_kernel(float* state, int64_t state_stride, const float* x, int64_t x_stride, const float* w, SeqBatch s, int width,
+                 float eps) {
+  __shared__ float red[kBlock / 64];
+  const int b = blockIdx.x;
+  int64_t start, len, prefix;
+  seq_span(s, b, start, len, prefix);
+  if (len <= 0) return;
+  const float* row = x + (start + len - 1) * x_stride;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < width; i += blockDim.x) ss += row[i] * row[i];
+  ss = block_sum(ss, red);
+  const float inv = 1.f / sqrtf(ss / (float)width + eps);
+  float* dst = state + load_idx(s.req_pool_indices, b, s.idx64) * state_stride;
+  for (int i = threadIdx.x; i < width; i += blockDim.x) dst[i] = row[i] * inv * w[i];
+}
+
+template <typename Tag>
+__global__ void stream_add_kernel(float* x, int64_t x_stride, const void* a, int64_t a_stride, const void* b, int64_t b_stride,
+                                  const void* c, int64_t c_stride, int width) {
+  typedef Elem<Tag> E;
+  const int64_t t = blockIdx.x;
+  for (int i = threadIdx.x; i < width; i += blockDim.x) {
+    float y = E::load(a, t * a_stride + i);
+    if (b) y += E::load(b, t * b_stride + i);
+    if (c) y += E::load(c, t * c_stride + i);
+    x[t * x_stride + i] += y;
+  }
+}
+
+}  // namespace
+}  // namespace sp
+
+using namespace sp;
+
+extern "C" int sp_embed_scale(float* x, int64_t x_stride, const void* embed, const int64_t* ids, int64_t num_tokens,
+                              int width, int64_t vocab, float scale, int dtype, void* stream) {
+  SP_CHECK_ARG(num_tokens >= 0 && width > 0 && vocab > 0);
+  if (num_tokens == 0) return SP_OK;
+  SP_CHECK_ARG(x && embed && ids && x_stride >= width);
+  SP_DISPATCH_DTYPE(dtype, (embed_scale_kernel<Tag><<<dim3((unsigned)num_tokens), kBlock, 0, (hipStream_t)stream>>>(
+                               x, x_stride, embed, ids, width, vocab, scale)));
+  SP_LAUNCH_CHECK();
+  return SP_OK;
+}
+
+extern "C" int sp_norm_shift(void* out_h, void* out_hs, int64_t out_stride, const float* x, int64_t x_stride,
+                             const float* weight, const float* mu, const float* state, int64_t state_stride,
+                             int64_t num_tokens, int width, float eps, SP_SEQ_PARAMS, int dtype, void* stream) {
+  SP_CHECK_ARG(num_tokens >= 0 && width > 0);
+  if (num_tokens == 0) return SP_OK;
+  SP_CHECK_ARG((out_h || out_hs) && x && weight && x_stride >= width && out_stride >= width);
+  if (out_hs) {
+    SP_CHECK_ARG(mu && state && state_stride >= width && req_pool_indices && seq_lens);
+    SP_CHECK_ARG(!extend_seq_lens || (extend_prefix_lens && extend_start_loc && token_req));
+    SP_CHECK_ARG(extend_seq_lens || num_tokens == batch_size);
+  }
+  SEQ_BATCH(s);
+  SP_DISPATCH_DTYPE(dtype, (norm_shift_kernel<Tag><<<dim3((unsigned)num_tokens), kBlock, 0, (hipStream_t)stream>>>(
+                               out_h, out_hs, out_stride, x, x_stride, weight, mu, state, state_stride, s, width, eps)));
+  SP_LAUNCH_CHECK();
+  return SP_OK;
+}
+
+extern "C" int sp_norm_save_last(float* state, int64_t state_stride, const float* x, int64_t x_stride, const float* weight,
+                                 int width, float eps, SP_SEQ_PARAMS, void* stream) {
+  SP_CHECK_ARG(batch_size >= 0 && width > 0);
+  if (batch_size == 0) return SP_OK;
+  SP_CHECK_ARG(state && x && weight && state_stride >= width && x_stride >= width && req_pool_indices && seq_lens);
+  SP_CHECK_ARG(!extend_seq_lens || (extend_prefix_lens && extend_start_loc));
+  SEQ_BATCH(s);
+  norm_save_kernel<<<dim3((unsigned)batch_size), kBlock, 0, (hipStream_t)stream>>>(state, state_stride, x, x_stride, weight,
+                                                                                  s, width, eps);
+  SP_LAUNCH_CHECK();
+  return SP_OK;
+}
+
+extern "C" int sp_stream_add(float* x, int64_t x_stride, const void* a, int64_t a_stride, const void* b, int64_t b_stride,
+                             const void* c, int64_t c_stride, int64_t num_tokens, int width, int dtype, void* stream) {
+  SP_CHECK_ARG(num_tokens >= 0 && width > 0);
+  if (num_tokens == 0) return SP_OK;
+  SP_CHECK_ARG(x && a && x_stride >= width && a_stride >= width && (!b || b_stride >= width) && (!c || c_stride >= width));
+  SP_DISPATCH_DTYPE(dtype, (stream_add_kernel<Tag><<<dim3((unsigned)num_tokens), kBlock, 0, (hipStream_t)stream>>>(
+                               x, x_stride, a, a_stride, b, b_stride, c, c_stride, width)));
+  SP_LAUNCH_CHECK();
+  return SP_OK;
+}

@@ -1,0 +1,259 @@
+// Grouped-query attention over a sliding window plus pooled blocks, on a token-level key/value pool.
+//
+// A query at position p sees the tokens j with 0 <= p - j < size and, for every block of P consecutive positions that
+// lies wholly before the window (block b = positions bP .. bP + P - 1, seen once bP + P - 1 <= p - size), ONE key and
+// value: the means of the block's cached keys and values.  Tokens and blocks share one softmax.  Tokens that left the
+// window while their block is still incomplete behind it are not seen.  size <= 0 means no window (plain causal),
+// P <= 0 no pooling.
+//
+// Cache: per token a key row [G, D] (rotated) and a value row [G, Dv] (each head divided by its root mean square); the
+// pooled key/value of block b lives in a second pair of buffers at the slot of the block's LAST token, written by the
+// step that brings this token, so the pooled rows need no allocator of their own and are freed with the token.
+//
+// Rotation: "rotate half" - coordinate i < dims/2 pairs with i + dims/2, angle = position * freq[i] in fp32, cos and
+// sin times mag; coordinates from dims on pass.  Scores, softmax and the weighted sum are fp32.
+#include "seq_batch.h"
+
+namespace sp {
+namespace {
+
+// q rotated in place; k rotated and v normed into the pool rows loc[t]
+template <typename Tag>
+__global__ void __launch_bounds__(kBlock)
+qkv_rotary_store_kernel(void* q, int64_t q_stride, const void* k, int64_t k_stride, const void* v, int64_t v_stride,
+                        void* kpool, int64_t kp_stride, void* vpool, int64_t vp_stride, const int64_t* positions,
+                        const int64_t* loc, const float* freq, float mag, int H, int G, int D, int Dv, int dims, float eps) {
+  typedef Elem<Tag> E;
+  const int64_t t = blockIdx.x;
+  const float pos = (float)positions[t];
+  const int half = dims / 2;
+  const int64_t slot = loc[t];
+  for (int e = threadIdx.x; e < H * half; e += blockDim.x) {
+    const int h = e / half, i = e % half;
+    const float a = pos * freq[i];
+    const float c = cosf(a) * mag, sn = sinf(a) * mag;
+    const int64_t at = t * q_stride + (int64_t)h * D + i;
+    const float u = E::load(q, at), w = E::load(q, at + half);
+    E::store(q, at, u * c - w * sn);
+    E::store(q, at + half, w * c + u * sn);
+  }
+  for (int e = threadIdx.x; e < G * half; e += blockDim.x) {
+    const int g = e / half, i = e % half;
+    const float a = pos * freq[i];
+    const float c = cosf(a) * mag, sn = sinf(a) * mag;
+    const int64_t at = t * k_stride + (int64_t)g * D + i, to = slot * kp_stride + (int64_t)g * D + i;
+    const float u = E::load(k, at), w = E::load(k, at + half);
+    E::store(kpool, to, u * c - w * sn);
+    E::store(kpool, to + half, w * c + u * sn);
+  }
+  const int rest = D - dims;
+  for (int e = threadIdx.x; e < G * rest; e += blockDim.x) {
+    const int g = e / rest, i = dims + e % rest;
+    E::store(kpool, slot * kp_stride + (int64_t)g * D + i, E::load(k, t * k_stride + (int64_t)g * D + i));
+  }
+  // value heads: one wave each
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, waves = blockDim.x >> 6;
+  for (int g = wave; g < G; g += waves) {
+    const int64_t at = t * v_stride + (int64_t)g * Dv, to = slot * vp_stride + (int64_t)g * Dv;
+    float ss = 0.f;
+    for (int i = lane; i < Dv; i += 64) {
+      const float x = E::load(v, at + i);
+      ss += x * x;
+    }
+    ss = wave_sum(ss);
+    const float inv = 1.f / sqrtf(ss / (float)Dv + eps);
+    for (int i = lane; i < Dv; i += 64) E::store(vpool, to + i, E::load(v, at + i) * inv);
+  }
+}
+
+// a token that completes a block (position + 1 divisible by P) writes the block's mean key and value at its own slot
+template <typename Tag>
+__global__ void __launch_bounds__(kBlock)
+pool_blocks_kernel(void* kpooled, void* vpooled, const void* kpool, const void* vpool, int64_t kp_stride, int64_t vp_stride,
+                   const int32_t* req_to_token, int64_t table_stride, SeqBatch s, int kw, int vw, int P) {
+  typedef Elem<Tag> E;
+  const int64_t t = blockIdx.x;
+  int b;
+  int64_t start, prefix;
+  seq_of_token(s, t, b, start, prefix);
+  const int64_t pos = prefix + (t - start);
+  if ((pos + 1) % P != 0) return;
+  const int32_t* table = req_to_token + load_idx(s.req_pool_indices, b, s.idx64) * table_stride;
+  const int64_t first = pos - P + 1, dst = table[pos];
+  const float inv = 1.f / (float)P;
+  for (int c = threadIdx.x; c < kw + vw; c += blockDim.x) {
+    const bool isk = c < kw;
+    const void* src = isk ? kpool : vpool;
+    const int64_t stride = isk ? kp_stride : vp_stride;
+    const int col = isk ? c : c - kw;
+    float acc = 0.f;
+    for (int j = 0; j < P; ++j) acc += E::load(src, (int64_t)table[first + j] * stride + col);
+    E::store(isk ? kpooled : vpooled, dst * stride + col, acc * inv);
+  }
+}
+
+constexpr int kMaxPerLane = 4;       // value width Dv <= 64 * kMaxPerLane
+
+template <typename Tag, bool VEC>
+__device__ __forceinline__ float dot_row(const float* sq, const void* base, int64_t at, int D) {
+  typedef Elem<Tag> E;
+  float d = 0.f;
+  if (VEC) {
+    constexpr int V = E::kVec;
+    for (int i = 0; i < D; i += V) {
+      float f[V];
+      unpack16<Tag>(ld16((const char*)base + (at + i) * E::kBytes), f);
+#pragma unroll
+      for (int e = 0; e < V; ++e) d += sq[i + e] * f[e];
+    }
+  } else {
+    for (int i = 0; i < D; ++i) d += sq[i] * E::load(base, at + i);
+  }
+  return d;
+}
+
+// One wave per (token, query head), 4 heads of a token per workgroup.  The query's keys are numbered blocks first, then
+// the window's tokens; tiles of 64: lane = key for the scores, lane = value channel for the weighted sum.
+template <typename Tag, bool VEC>
+__global__ void __launch_bounds__(256)
+window_attention_kernel(void* out, int64_t out_stride, const void* q, int64_t q_stride, const void* kpool, const void* vpool,
+                        const void* kpooled, const void* vpooled, int64_t kp_stride, int64_t vp_stride,
+                        const int32_t* req_to_token, int64_t table_stride, SeqBatch s, int H, int G, int D, int Dv,
+                        int64_t size, int P, float scale) {
+  typedef Elem<Tag> E;
+  extern __shared__ float smem[];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int64_t t = blockIdx.x;
+  const int h = blockIdx.y * 4 + wave;
+  if (h >= H) return;                                    // (no workgroup barrier below)
+  float* sq = smem + (size_t)wave * (D + 64);
+  float* sw = sq + D;
+  int b;
+  int64_t start, prefix;
+  seq_of_token(s, t, b, start, prefix);
+  const int64_t pos = prefix + (t - start);
+  const int64_t w0 = (size > 0 && pos - size + 1 > 0) ? pos - size + 1 : 0;      // first token of the window
+  const int64_t nb = (size > 0 && P > 0) ? w0 / P : 0;                            // blocks wholly before it
+  const int64_t total = nb + (pos - w0 + 1);
+  const int g = h / (H / G);
+  const int32_t* table = req_to_token + load_idx(s.req_pool_indices, b, s.idx64) * table_stride;
+  for (int i = lane; i < D; i += 64) sq[i] = E::load(q, t * q_stride + (int64_t)h * D + i) * scale;
+  __builtin_amdgcn_wave_barrier();
+  float m = -INFINITY, l = 0.f;
+  float acc[kMaxPerLane];
+#pragma unroll
+  for (int i = 0; i < kMaxPerLane; ++i) acc[i] = 0.f;
+  for (int64_t k0 = 0; k0 < total; k0 += 64) {
+    const int n = (int)(total - k0 < 64 ? total - k0 : 64);
+    float sc = -INFINITY;
+    if (lane < n) {
+      const int64_t kk = k0 + lane;
+      const bool blk = kk < nb;
+      const int64_t row = blk ? table[kk * P + P - 1] : table[w0 + (kk - nb)];
+      sc = dot_row<Tag, VEC>(sq, blk ? kpooled : kpool, row * kp_stride + (int64_t)g * D, D);
+    }
+    float tm = sc;
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) tm = fmaxf(tm, __shfl_xor(tm, off, 64));
+    const float m_new = fmaxf(m, tm);
+    const float corr = expf(m - m_new);                 // first tile: exp(-inf) = 0
+    const float p = lane < n ? expf(sc - m_new) : 0.f;
+    l = l * corr + wave_sum(p);
+    m = m_new;
+    sw[lane] = p;
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int i = 0; i < kMaxPerLane; ++i) acc[i] *= corr;
+    for (int j = 0; j < n; ++j) {
+      const int64_t kk = k0 + j;
+      const bool blk = kk < nb;
+      const int64_t row = blk ? table[kk * P + P - 1] : table[w0 + (kk - nb)];
+      const void* src = blk ? vpooled : vpool;
+      const float pj = sw[j];
+#pragma unroll
+      for (int i = 0; i < kMaxPerLane; ++i) {
+        const int c = lane + 64 * i;
+        if (c < Dv) acc[i] += pj * E::load(src, row * vp_stride + (int64_t)g * Dv + c);
+      }
+    }
+    __builtin_amdgcn_wave_barrier();
+  }
+  const float inv = 1.f / l;
+#pragma unroll
+  for (int i = 0; i < kMaxPerLane; ++i) {
+    const int c = lane + 64 * i;
+    if (c < Dv) E::store(out, t * out_stride + (int64_t)h * Dv + c, acc[i] * inv);
+  }
+}
+
+}  // namespace
+}  // namespace sp
+
+using namespace sp;
+
+extern "C" int sp_qkv_rotary_store(void* q, int64_t q_stride, const void* k, int64_t k_stride, const void* v,
+                                   int64_t v_stride, void* kpool, int64_t kp_stride, void* vpool, int64_t vp_stride,
+                                   const int64_t* positions, const int64_t* loc, const float* freq, float mag,
+                                   int64_t num_tokens, int heads, int kv_heads, int dim, int vdim, int rot_dims, float eps,
+                                   int dtype, void* stream) {
+  SP_CHECK_ARG(num_tokens >= 0 && heads > 0 && kv_heads > 0 && dim > 0 && vdim > 0);
+  SP_CHECK_ARG(rot_dims >= 0 && rot_dims % 2 == 0 && rot_dims <= dim);
+  if (num_tokens == 0) return SP_OK;
+  SP_CHECK_ARG(q && k && v && kpool && vpool && positions && loc && (freq || rot_dims == 0));
+  SP_CHECK_ARG(q_stride >= (int64_t)heads * dim && k_stride >= (int64_t)kv_heads * dim && v_stride >= (int64_t)kv_heads * vdim);
+  SP_CHECK_ARG(kp_stride >= (int64_t)kv_heads * dim && vp_stride >= (int64_t)kv_heads * vdim);
+  SP_DISPATCH_DTYPE(dtype, (qkv_rotary_store_kernel<Tag><<<dim3((unsigned)num_tokens), kBlock, 0, (hipStream_t)stream>>>(
+                               q, q_stride, k, k_stride, v, v_stride, kpool, kp_stride, vpool, vp_stride, positions, loc,
+                               freq, mag, heads, kv_heads, dim, vdim, rot_dims, eps)));
+  SP_LAUNCH_CHECK();
+  return SP_OK;
+}
+
+extern "C" int sp_pool_blocks(void* kpooled, void* vpooled, const void* kpool, const void* vpool, int64_t kp_stride,
+                              int64_t vp_stride, const int32_t* req_to_token, int64_t table_stride, int64_t num_tokens,
+                              int key_width, int value_width, int block, SP_SEQ_PARAMS, int dtype, void* stream) {
+  SP_CHECK_ARG(num_tokens >= 0 && key_width > 0 && value_width > 0 && block > 0);
+  if (num_tokens == 0) return SP_OK;
+  SP_CHECK_ARG(kpooled && vpooled && kpool && vpool && req_to_token && req_pool_indices && seq_lens);
+  SP_CHECK_ARG(kp_stride >= key_width && vp_stride >= value_width);
+  SP_CHECK_ARG(!extend_seq_lens || (extend_prefix_lens && extend_start_loc && token_req));
+  SP_CHECK_ARG(extend_seq_lens || num_tokens == batch_size);
+  SEQ_BATCH(s);
+  SP_DISPATCH_DTYPE(dtype, (pool_blocks_kernel<Tag><<<dim3((unsigned)num_tokens), kBlock, 0, (hipStream_t)stream>>>(
+                               kpooled, vpooled, kpool, vpool, kp_stride, vp_stride, req_to_token, table_stride, s, key_width,
+                               value_width, block)));
+  SP_LAUNCH_CHECK();
+  return SP_OK;
+}
+
+extern "C" int sp_window_attention(void* out, int64_t out_stride, const void* q, int64_t q_stride, const void* kpool,
+                                   const void* vpool, const void* kpooled, const void* vpooled, int64_t kp_stride,
+                                   int64_t vp_stride, const int32_t* req_to_token, int64_t table_stride,
+                                   int64_t num_tokens, int heads, int kv_heads, int dim, int vdim, int64_t window, int block,
+                                   float scale, SP_SEQ_PARAMS, int dtype, void* stream) {
+  SP_CHECK_ARG(num_tokens >= 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0 && dim > 0 && vdim > 0);
+  if (num_tokens == 0) return SP_OK;
+  SP_CHECK_ARG(out && q && kpool && vpool && req_to_token && req_pool_indices && seq_lens);
+  SP_CHECK_ARG((kpooled && vpooled) || block <= 0 || window <= 0);
+  SP_CHECK_ARG(!extend_seq_lens || (extend_prefix_lens && extend_start_loc && token_req));
+  SP_CHECK_ARG(extend_seq_lens || num_tokens == batch_size);
+  SP_CHECK_ARG(q_stride >= (int64_t)heads * dim && out_stride >= (int64_t)heads * vdim);
+  SP_CHECK_ARG(kp_stride >= (int64_t)kv_heads * dim && vp_stride >= (int64_t)kv_heads * vdim);
+  if (vdim > 64 * kMaxPerLane) return SP_ERR_UNSUPPORTED;
+  const size_t lds = 4 * (size_t)(dim + 64) * sizeof(float);
+  if (lds > 64 * 1024) return SP_ERR_UNSUPPORTED;
+  SEQ_BATCH(s);
+  const dim3 grid((unsigned)num_tokens, (unsigned)((heads + 3) / 4));
+  const int vecn = dtype == SP_F32 ? 4 : 8;
+  const bool vec = dim % vecn == 0 && kp_stride % vecn == 0 && ((uintptr_t)kpool & 15) == 0 &&
+                   (!kpooled || ((uintptr_t)kpooled & 15) == 0);
+#define SP_WA(V)                                                                                                       \
+  SP_DISPATCH_DTYPE(dtype, (window_attention_kernel<Tag, V><<<grid, 256, lds, (hipStream_t)stream>>>(                   \
+                               out, out_stride, q, q_stride, kpool, vpool, kpooled, vpooled, kp_stride, vp_stride,      \
+                               req_to_token, table_stride, s, heads, kv_heads, dim, vdim, window, block, scale)))
+  if (vec) SP_WA(true);
+  else SP_WA(false);
+#undef SP_WA
+  SP_LAUNCH_CHECK();
+  return SP_OK;
+}

@@ -285,3 +285,48 @@ class AngleRotary(nn.Module):
     def forward(self, positions: torch.Tensor, x: torch.Tensor, offset: int = 0) -> None:
         """in place on x [T, H, n]: coordinates offset .. offset + dims of every head"""
         _native.rotary_interleaved(x, positions, self.freq, self.magnitude, offset)
+
+
+class HalfAngleRotary(AngleRotary):
+    """The same fp32 frequencies and magnitude, for the "rotate half" pairing: coordinate i < dims / 2 pairs with
+    i + dims / 2.  Applied by the fused rotation + cache store (_native.qkv_rotary_store), not by a call of its own."""
+
+    def forward(self, positions: torch.Tensor, x: torch.Tensor, offset: int = 0) -> None:
+        raise NotImplementedError("the half-pair rotation runs inside _native.qkv_rotary_store")
+
+
+class ShiftedRMSNorm(nn.Module):
+    """Weighted RMS norm of an fp32 residual stream followed by a token shift: h = x / rms(x) * weight is what a layer's
+    feed-forward reads, hs = h + (h[t-1] - h) * mu what its mixer reads; h[t-1] before a step's first row is the request's
+    saved h (RecurrentStatePool.shift_state; zeros for a sequence's first token).  Both come out in the projections'
+    dtype; the arithmetic and the saved row are fp32.  Without ``shift`` it is a plain weighted norm (a model's last)."""
+
+    def __init__(self, width: int, eps: float = 1e-6, shift: bool = True, layer_id: Optional[int] = None) -> None:
+        super().__init__()
+        self.weight = nn.Parameter(torch.ones(width, dtype=torch.float32), requires_grad=False)
+        self.mu = nn.Parameter(torch.zeros(width, dtype=torch.float32), requires_grad=False) if shift else None
+        self.variance_epsilon, self.layer_id = eps, layer_id
+
+    def forward(self, x: torch.Tensor, dtype: torch.dtype, forward_batch=None, want_h: bool = True):
+        if self.mu is None:
+            return _native.norm_shift(x, self.weight.data, self.variance_epsilon, dtype)[0]
+        return _native.norm_shift(x, self.weight.data, self.variance_epsilon, dtype, self.mu.data,
+                                  forward_batch.state_pool.shift_state(self.layer_id), forward_batch.attn_backend.seq, want_h)
+
+
+class GluFF(nn.Module):
+    """Gated feed-forward with the gate and up projections as ONE product: act = "silu": W_down (silu(g) * u);
+    act = "clamped": g' = min(g, limit), u' = clamp(u, -limit, limit), W_down (g' * sigmoid(alpha g') * (u' + 1))."""
+
+    def __init__(self, width: int, ff: int, act: str = "silu", limit: float = 0.0, alpha: float = 1.702, dtype=None):
+        super().__init__()
+        if act not in ("silu", "clamped"):
+            raise ValueError(f"unknown activation {act!r}")
+        self.ff, self.act, self.limit, self.alpha = ff, act, limit, alpha
+        self.gate_up = nn.Parameter(torch.empty(2 * ff, width, dtype=dtype), requires_grad=False)
+        self.down = nn.Parameter(torch.empty(width, ff, dtype=dtype), requires_grad=False)
+
+    def forward(self, h: torch.Tensor) -> torch.Tensor:
+        gu = _native.linear(h, self.gate_up)
+        y = _native.silu_and_mul(gu) if self.act == "silu" else _native.moe_glu(gu.contiguous(), self.limit, self.alpha)
+        return _native.linear(y, self.down)

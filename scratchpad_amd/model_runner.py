@@ -195,6 +195,18 @@ class ModelRunner:
                                2048), 4096)
         self.max_running_requests = max_reqs
         self.state_pool = None
+        if hasattr(self.model_config, "window_cache"):
+            # windowed key/value rows for the attention layers, named per-request state (and a shift row) for the others;
+            # request row 0 is kept back for the padded rows of a graph replay
+            from .pool import WindowKVPool
+            cfg = self.model_config
+            self.req_to_token_pool = ReqToTokenPool(max_reqs + 1, cfg.context_len + 4, self.device, reserved_rows=1)
+            self.token_to_kv_pool = WindowKVPool(self.max_total_num_tokens, self.kv_cache_dtype, cfg.window_cache(), self.device)
+            self.state_pool = RecurrentStatePool(max_reqs + 1, cfg.hidden_size, {}, self.device,
+                                                 shift_layers=cfg.shift_layers(), named=cfg.named_state())
+            self.token_to_kv_pool_allocator = TokenToKVPoolAllocator(
+                self.max_total_num_tokens, self.kv_cache_dtype, self.device, self.token_to_kv_pool)
+            return
         if hasattr(self.model_config, "latent_cache"):
             # latent key/value rows for the attention layers, per-request state for the recurrent ones; request row 0 is
             # kept back for the padded rows of a graph replay (they must not touch a live request's state)

@@ -31,12 +31,15 @@ class ClampedGluExperts(nn.Module):
         self.gate_up = nn.Parameter(torch.empty(experts, 2 * ff, width, dtype=dtype), requires_grad=False)
         self.down = nn.Parameter(torch.empty(experts, width, ff, dtype=dtype), requires_grad=False)
 
+    def activation(self, gu: torch.Tensor) -> torch.Tensor:
+        return _native.moe_glu(gu, self.limit, self.alpha)
+
     def forward(self, x: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor) -> torch.Tensor:
         top = ids.shape[1]
         pairs = ids.numel()
         offsets, order, place = _native.moe_align(ids, self.experts)
         gu = _native.moe_grouped_gemm(x, self.gate_up.data, offsets, pairs, order, top)
-        y = _native.moe_glu(gu, self.limit, self.alpha)
+        y = self.activation(gu)
         z = _native.moe_grouped_gemm(y, self.down.data, offsets, pairs)
         return _native.moe_combine(z, place, weights)
 
@@ -47,6 +50,43 @@ class SparseMoE(nn.Module):
         super().__init__()
         self.router = GroupLimitedRouter(width, experts, top, groups, keep)
         self.experts = ClampedGluExperts(width, experts, ff, limit, dtype=dtype)
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        ids, weights = self.router(x)
+        return self.experts(x, ids, weights)
+
+
+class SoftmaxRouter(nn.Module):
+    """ids, weights = the `top` experts with the largest softmax(W x) over ALL experts (fp32 logits); the weights are
+    those scores times `scale`, not renormalised over the chosen ones."""
+
+    def __init__(self, width: int, experts: int, top: int, scale: float = 1.0):
+        super().__init__()
+        self.experts, self.top, self.scale = experts, top, scale
+        self.weight = nn.Parameter(torch.zeros(experts, width, dtype=torch.float32), requires_grad=False)
+
+    def forward(self, x: torch.Tensor):
+        return _native.moe_route_softmax(x, self.weight.data, self.top, self.scale)
+
+
+class SiluGluExperts(ClampedGluExperts):
+    """Experts y = W_down (silu(W_gate x) * (W_up x)): the same stacked layout and grouped products, no clamps."""
+
+    def __init__(self, width: int, experts: int, ff: int, dtype=None):
+        super().__init__(width, experts, ff, 0.0, dtype=dtype)
+
+    def activation(self, gu: torch.Tensor) -> torch.Tensor:
+        return _native.silu_and_mul(gu)
+
+
+class SoftmaxMoE(nn.Module):
+    """SoftmaxRouter + SiluGluExperts; `forward` returns the routed experts' weighted sum (a shared expert, if the model
+    has one, is a dense feed-forward of its own beside this)."""
+
+    def __init__(self, width: int, experts: int, top: int, ff: int, scale: float = 1.0, dtype=None):
+        super().__init__()
+        self.router = SoftmaxRouter(width, experts, top, scale)
+        self.experts = SiluGluExperts(width, experts, ff, dtype=dtype)
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         ids, weights = self.router(x)

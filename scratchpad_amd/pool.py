@@ -434,6 +434,64 @@ class LatentTokenToKVPool(KVCache):
         self._buffers[layer_id][indices] = flat_data.to(device=self.device, non_blocking=False)
 
 
+class WindowKVPool(KVCache):
+    """Token-level key/value pool whose layers differ in width and whose key and value widths differ: per layer in
+    ``layers`` ({layer id: (kv_heads, dim, vdim, pooled)}) a key buffer [P+1, kv_heads * dim] and a value buffer
+    [P+1, kv_heads * vdim]; layers with ``pooled`` also get a second pair of the same shape that holds, at the slot of a
+    block's last token, the mean key and value of the block (attention.PooledWindowAttention).  Same slot ids, allocator
+    and dummy slot 0 as MHATokenToKVPool; layers not named take no memory."""
+
+    def __init__(self, size: int, dtype: torch.dtype, layers, device: str):
+        if dtype not in (torch.float32, torch.float16, torch.bfloat16):
+            raise NotImplementedError(f"window KV cache dtype {dtype} is not built")
+        self.size, self.page_size, self.dtype, self.store_dtype, self.device = size, 1, dtype, dtype, device
+        self.layers = {int(l): (int(g), int(d), int(dv), bool(p)) for l, (g, d, dv, p) in layers.items()}
+        z = lambda n: torch.zeros((size + 1, n), dtype=dtype, device=device)
+        self._k = {l: z(g * d) for l, (g, d, dv, p) in self.layers.items()}
+        self._v = {l: z(g * dv) for l, (g, d, dv, p) in self.layers.items()}
+        self._kp = {l: z(g * d) for l, (g, d, dv, p) in self.layers.items() if p}
+        self._vp = {l: z(g * dv) for l, (g, d, dv, p) in self.layers.items() if p}
+        self.layer_num = len(self.layers)
+        self.layer_transfer_counter = None
+
+    def _all(self):
+        return [b[l] for l in sorted(self.layers) for b in (self._k, self._v, self._kp, self._vp) if l in b]
+
+    def get_kv_size_bytes(self):
+        return (sum(b.nbytes for d in (self._k, self._kp) for b in d.values()),
+                sum(b.nbytes for d in (self._v, self._vp) for b in d.values()))
+
+    def get_key_buffer(self, layer_id: int) -> torch.Tensor:
+        return self._k[layer_id]
+
+    def get_value_buffer(self, layer_id: int) -> torch.Tensor:
+        return self._v[layer_id]
+
+    def get_kv_buffer(self, layer_id: int):
+        return self._k[layer_id], self._v[layer_id]
+
+    def get_pooled_buffers(self, layer_id: int):
+        """(keys, values) of the blocks, or (None, None) for a layer without pooling"""
+        return self._kp.get(layer_id), self._vp.get(layer_id)
+
+    def set_kv_buffer(self, layer, loc: torch.Tensor, cache_k: torch.Tensor, cache_v: torch.Tensor) -> None:
+        """rows already rotated / normed (the fused store, _native.qkv_rotary_store, is what the model path runs)"""
+        self._k[layer.layer_id][loc] = cache_k.reshape(loc.shape[0], -1).to(self.dtype)
+        self._v[layer.layer_id][loc] = cache_v.reshape(loc.shape[0], -1).to(self.dtype)
+
+    def get_flat_data(self, indices):
+        return [b[indices] for b in self._all()]
+
+    def transfer(self, indices, flat_data):
+        for b, data in zip(self._all(), flat_data):
+            b[indices] = data.to(device=self.device, non_blocking=False)
+
+    def transfer_per_layer(self, indices, flat_data, layer_id):
+        bufs = [b[layer_id] for b in (self._k, self._v, self._kp, self._vp) if layer_id in b]
+        for b, data in zip(bufs, flat_data):
+            b[indices] = data.to(device=self.device, non_blocking=False)
+
+
 class RecurrentStatePool:
     """Per-request state of models whose layers carry something from token to token besides a key/value cache: one slot
     per row of the ReqToTokenPool (the request's row index IS its state slot, so admission, release and reuse of a slot
@@ -442,24 +500,36 @@ class RecurrentStatePool:
     * ``last_token`` [slots] int64: the request's latest token (input of a hashed previous-token embedding);
     * per recurrent layer ``shift`` [slots, width] (the layer input of the latest token, for the token shift) and
       ``matrix`` [slots, heads, dim, dim] (the recurrence's state);
+    * per layer any further named tensors [slots, ...] (a non-square matrix memory, its normaliser and running maximum, a
+      convolution's latest inputs); a model may also ask for shift rows in layers without a matrix state;
     * nothing is cleared when a slot changes hands: every kernel starts a request that holds no token yet from the initial
       state, whatever the slot contains.  Row 0 belongs to the padded rows of a graph replay (ReqToTokenPool.reserved_rows)."""
 
-    def __init__(self, slots: int, width: int, layers, device: str):
-        """layers: {layer_id: (heads, dim)} of the recurrent layers"""
+    def __init__(self, slots: int, width: int, layers, device: str, shift_layers=None, named=None):
+        """layers: {layer_id: (heads, dim)} of the layers with a square matrix state; shift_layers: ids of the layers
+        that keep their previous input row (default: those of ``layers``); named: {layer_id: {name: shape}} further fp32
+        state tensors, each [slots, *shape] (``state(layer_id, name)``)"""
         self.slots, self.width, self.device = slots, width, device
         self.layer_ids = sorted(layers)
         self._index = {l: i for i, l in enumerate(self.layer_ids)}
+        shift_ids = self.layer_ids if shift_layers is None else sorted(shift_layers)
+        self._shift_index = {l: i for i, l in enumerate(shift_ids)}
         self.last_token = torch.zeros(slots, dtype=torch.int64, device=device)
-        self.shift = torch.zeros((len(self.layer_ids), slots, width), dtype=torch.float32, device=device)
+        self.shift = torch.zeros((len(shift_ids), slots, width), dtype=torch.float32, device=device)
         self.matrix = [torch.zeros((slots, h, d, d), dtype=torch.float32, device=device)
                        for h, d in (layers[l] for l in self.layer_ids)]
+        self.named = {int(l): {name: torch.zeros((slots, *shape), dtype=torch.float32, device=device)
+                               for name, shape in spec.items()} for l, spec in (named or {}).items()}
 
     def shift_state(self, layer_id: int) -> torch.Tensor:
-        return self.shift[self._index[layer_id]]
+        return self.shift[self._shift_index[layer_id]]
+
+    def state(self, layer_id: int, name: str) -> torch.Tensor:
+        return self.named[layer_id][name]
 
     def matrix_state(self, layer_id: int) -> torch.Tensor:
         return self.matrix[self._index[layer_id]]
 
     def size_bytes(self) -> int:
-        return self.last_token.nbytes + self.shift.nbytes + sum(m.nbytes for m in self.matrix)
+        return (self.last_token.nbytes + self.shift.nbytes + sum(m.nbytes for m in self.matrix) +
+                sum(t.nbytes for spec in self.named.values() for t in spec.values()))

@@ -1,4 +1,7 @@
-"""Recurrent token mixer with a per-head matrix state (RWKV-style time mixing) over the HIP kernels of csrc/wkv.hip.
+"""Recurrent token mixers over per-request state in the RecurrentStatePool: WKVMixer (RWKV-style time mixing, csrc/wkv.hip),
+Mamba2Mixer (state-space duality form, csrc/ssm.hip) and MLSTMMixer (matrix memory with exponential gating, csrc/mlstm.hip).
+
+WKVMixer:
 
 Per token t with layer input h[t] (the fp32 residual stream) and h[t-1] (zeros at a sequence's first token):
   m_s = h[t] + (h[t-1] - h[t]) * mu_s                      one mix per projection s in (r, k, v, g, w)
@@ -42,4 +45,82 @@ class WKVMixer(nn.Module):
         decay = _native.wkv_decay(_native.linear(mixes[4], self.w1), self.w2t.data, self.w0.data)
         o = _native.wkv_recurrence(rkvg[0], rkvg[1], rkvg[2], rkvg[3], decay, self.u.data, self.norm.data,
                                    states.matrix_state(self.layer_id), seq, self.heads, self.dim, self.eps)
+        return _native.linear(o, self.o)
+
+
+class Mamba2Mixer(nn.Module):
+    """State-space mixer.  With inner = heads * vdim, N = state, G = groups, the input projection's rows are
+    [z: inner | x: inner | B: G N | C: G N | dt: heads]; x, B, C pass a causal per-channel convolution (its latest
+    taps - 1 inputs are request state) and silu; per head h (group h // (heads / G)), in fp32:
+      dt = softplus(dt + dt_bias)    S <- exp(-exp(A_log) dt) S + dt B x^T    y = S^T C + D x        (S [N, vdim])
+    then out = W_o (groupnorm(y * silu(z)) * norm): the gate before the norm, ``norm_groups`` equal parts.
+    The dt rows of the projection are kept apart in fp32 (a step size is never rounded to 16 bits)."""
+
+    def __init__(self, width: int, heads: int, vdim: int, state: int, groups: int, taps: int, norm_groups: int,
+                 layer_id: int, eps: float, dtype=None):
+        super().__init__()
+        if heads % groups or (heads * vdim) % norm_groups:
+            raise ValueError("heads must divide into groups, heads * vdim into norm_groups")
+        self.heads, self.vdim, self.state, self.groups, self.taps = heads, vdim, state, groups, taps
+        self.norm_groups, self.layer_id, self.eps = norm_groups, layer_id, eps
+        inner, ch = heads * vdim, heads * vdim + 2 * groups * state
+        f32 = dict(dtype=torch.float32)
+        self.in_proj = nn.Parameter(torch.empty(inner + ch, width, dtype=dtype), requires_grad=False)     # [z | x | B | C]
+        self.dt_proj = nn.Parameter(torch.zeros(heads, width, **f32), requires_grad=False)
+        self.conv = nn.Parameter(torch.zeros(ch, taps, **f32), requires_grad=False)
+        self.conv_bias = nn.Parameter(torch.zeros(ch, **f32), requires_grad=False)
+        self.dt_bias = nn.Parameter(torch.zeros(heads, **f32), requires_grad=False)
+        self.A_log = nn.Parameter(torch.zeros(heads, **f32), requires_grad=False)
+        self.D = nn.Parameter(torch.ones(heads, **f32), requires_grad=False)
+        self.norm = nn.Parameter(torch.ones(inner, **f32), requires_grad=False)
+        self.o = nn.Parameter(torch.empty(width, inner, dtype=dtype), requires_grad=False)
+
+    @staticmethod
+    def state_shapes(heads: int, vdim: int, state: int, groups: int, taps: int):
+        return {"ssm": (heads, state, vdim), "conv": (max(taps - 1, 0), heads * vdim + 2 * groups * state)}
+
+    def forward(self, h: torch.Tensor, forward_batch: ForwardBatch) -> torch.Tensor:
+        seq, states = forward_batch.attn_backend.seq, forward_batch.state_pool
+        inner = self.heads * self.vdim
+        zxbc = _native.linear(h, self.in_proj)
+        dt = _native.small_linear_f32(h, self.dt_proj.data)
+        xbc = _native.causal_conv_silu(zxbc[:, inner:], self.conv.data, self.conv_bias.data,
+                                       states.state(self.layer_id, "conv"), seq)
+        y = _native.mamba2_scan(xbc, dt, self.dt_bias.data, self.A_log.data, self.D.data, states.state(self.layer_id, "ssm"),
+                                seq, self.heads, self.groups, self.state, self.vdim)
+        return _native.linear(_native.gated_group_norm(y, zxbc[:, :inner], self.norm.data, self.norm_groups, self.eps), self.o)
+
+
+class MLSTMMixer(nn.Module):
+    """Matrix-memory mixer with exponential gating.  q, k [heads, dim], v [heads, vdim], an output gate g and, per head, a
+    log input gate i = cap tanh((W_i h + b_i) / cap) and a log forget gate f = logsigmoid(cap tanh((W_f h + b_f) / cap));
+    with a running maximum m (0 for a new sequence):  m' = max(f + m, i),  S <- exp(f + m - m') S + exp(i - m') k v^T,
+    n likewise with k,  o = S^T q / (max(|n . q|, exp(-m')) + 1e-6) with q scaled by dim^(-1/2);
+    out = W_o (o / rms_head(o) * norm * sigmoid(g)).  q, k, v, g come from ONE product; the gate rows are a separate fp32
+    product (a gate is never rounded to 16 bits)."""
+
+    def __init__(self, width: int, heads: int, dim: int, vdim: int, gate_cap: float, layer_id: int, eps: float, dtype=None):
+        super().__init__()
+        self.heads, self.dim, self.vdim, self.cap, self.layer_id, self.eps = heads, dim, vdim, gate_cap, layer_id, eps
+        f32 = dict(dtype=torch.float32)
+        self.qkvg = nn.Parameter(torch.empty(2 * heads * dim + 2 * heads * vdim, width, dtype=dtype), requires_grad=False)
+        self.gates = nn.Parameter(torch.zeros(2 * heads, width, **f32), requires_grad=False)       # [i rows | f rows]
+        self.gates_bias = nn.Parameter(torch.zeros(2 * heads, **f32), requires_grad=False)
+        self.norm = nn.Parameter(torch.ones(heads * vdim, **f32), requires_grad=False)
+        self.o = nn.Parameter(torch.empty(width, heads * vdim, dtype=dtype), requires_grad=False)
+
+    @staticmethod
+    def state_shapes(heads: int, dim: int, vdim: int):
+        return {"S": (heads, dim, vdim), "n": (heads, dim), "m": (heads,)}
+
+    def forward(self, h: torch.Tensor, forward_batch: ForwardBatch) -> torch.Tensor:
+        seq, states = forward_batch.attn_backend.seq, forward_batch.state_pool
+        nk, nv, H = self.heads * self.dim, self.heads * self.vdim, self.heads
+        a = _native.linear(h, self.qkvg)
+        gates = _native.small_linear_f32(h, self.gates.data, self.gates_bias.data)
+        ipre, fpre = gates[:, :H].contiguous(), gates[:, H:].contiguous()
+        L = self.layer_id
+        o = _native.mlstm_scan(a[:, :nk], a[:, nk:2 * nk], a[:, 2 * nk:2 * nk + nv], a[:, 2 * nk + nv:], ipre, fpre,
+                               self.norm.data, states.state(L, "S"), states.state(L, "n"), states.state(L, "m"), seq,
+                               self.heads, self.dim, self.vdim, self.cap, self.eps)
         return _native.linear(o, self.o)

@@ -30,6 +30,11 @@ def _tizalorn_config(raw: dict, context_len=None, tensor_shapes=None, **_kw):
     return TizalornConfig(raw, context_len=context_len or 8192, tensor_shapes=tensor_shapes)
 
 
+def _sominex_config(raw: dict, context_len=None, tensor_shapes=None, **_kw):
+    from .sominex import SominexConfig
+    return SominexConfig(raw, context_len=context_len or 8192, tensor_shapes=tensor_shapes)
+
+
 def _llama_class():
     from .llama import LlamaForCausalLM
     return LlamaForCausalLM
@@ -45,11 +50,17 @@ def _tizalorn_class():
     return TizalornForCausalLM
 
 
+def _sominex_class():
+    from .sominex import SominexForCausalLM
+    return SominexForCausalLM
+
+
 # architecture name -> (configuration from config.json's dict, model class); both lazy so that naming a model does not
 # import the others
 MODELS = {
     "LlamaForCausalLM": (_llama_config, _llama_class),
     "Tizalorn": (_tizalorn_config, _tizalorn_class),
+    "Sominex": (_sominex_config, _sominex_class),
 }
 
 
