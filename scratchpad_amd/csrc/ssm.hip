@@ -189,8 +189,9 @@ extern "C" int sp_causal_conv_silu(void* out, int64_t out_stride, const void* in
                                    int taps, SP_SEQ_PARAMS, int dtype, void* stream) {
   SP_CHECK_ARG(num_tokens >= 0 && channels > 0 && taps >= 1 && taps <= kMaxTaps);
   if (num_tokens == 0) return SP_OK;
-  SP_CHECK_ARG(out && in && weight && state && req_pool_indices && seq_lens);
-  SP_CHECK_ARG(out_stride >= channels && in_stride >= channels && state_stride >= (int64_t)(taps - 1) * channels);
+  SP_CHECK_ARG(out && in && weight && req_pool_indices && seq_lens);
+  SP_CHECK_ARG(out_stride >= channels && in_stride >= channels);
+  SP_CHECK_ARG(taps == 1 || (state && state_stride >= (int64_t)(taps - 1) * channels));      // one tap: nothing is carried
   SP_CHECK_ARG(!extend_seq_lens || (extend_prefix_lens && extend_start_loc && token_req));
   SP_CHECK_ARG(extend_seq_lens || num_tokens == batch_size);
   SEQ_BATCH(s);

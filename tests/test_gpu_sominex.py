@@ -212,8 +212,11 @@ def test_whole_prompt_and_every_layer(full):
 
 def test_bf16_serving_precision(full):
     cfg, folder, w, toks, want, _ = full
-    got = run_portions(engine(folder, dtype=torch.bfloat16), toks, [40, 1])
-    assert U.rel(got, want) < 0.08
+    got = run_portions(engine(folder, dtype=torch.bfloat16), toks, [40, 1]).double().cpu()
+    # per position: rms of the deviation over the vocabulary against the rms of the logits.  16-bit rounding may flip a
+    # close expert choice at a position, so the bar is on the bulk of the positions, with a cap on the rest.
+    err = ((got - want) ** 2).mean(-1).sqrt() / (want ** 2).mean(-1).sqrt()
+    assert float(err.median()) < 0.03 and float((err > 0.15).double().mean()) <= 0.05 and float(err.max()) < 0.6, err
 
 
 @pytest.mark.parametrize("graphs", [False, True], ids=["eager", "graphs"])
