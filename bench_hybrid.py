@@ -1,5 +1,5 @@
-"""bench.py --mode hybrid: prefill and decode throughput of the Tizalorn design at layer sizes of real models (random
-weights), beside a Llama of the same width and depth on the same engine path, and a per-kernel table: every HIP kernel
+"""bench.py --mode hybrid / --mode sominex: prefill and decode throughput of the Tizalorn / the Sominex design at layer sizes
+of real models (random weights), beside a Llama of the same width and depth on the same engine path, and a per-kernel table: every HIP kernel
 (and library product) of both models timed inside an eager prefill batch and an eager decode step, with the time its
 algorithmic bytes and flops would take at the chip's peaks (fraction of roofline).
 
@@ -15,7 +15,7 @@ HBM = 8.0e12            # bytes/s
 MATRIX = 2.5e15         # dense bf16 flops/s on the matrix cores
 VECTOR32 = 157.3e12     # fp32 flops/s on the vector units (kernels whose arithmetic is fp32 by contract)
 
-SIZES = {"m": 2048, "l": 4096}      # widths of Llama-3.2-1B and Llama-3-8B, whose layers are the comparison
+SIZES = {"s": 1024, "m": 2048, "l": 4096}      # widths of Llama-3.2-1B and Llama-3-8B, whose layers are the comparison
 # Decode steps are launched eagerly for both models unless --graph is given.
 
 
@@ -36,10 +36,32 @@ def tizalorn_config(width: int, layers: int, context_len: int):
     return TizalornConfig(raw, context_len=context_len)
 
 
+def sominex_config(width: int, layers: int, context_len: int):
+    """layers in the order attention, mamba2, mlstm, mlstm with dense and expert feed-forwards alternating; head sizes of
+    128, a window of 512 tokens with blocks of 64 behind it, state 128, 32 experts of which 4 (+ a shared one)"""
+    from scratchpad_amd.sominex import SominexConfig
+    att = {"type": "attention",
+           "mixer": {"heads": width // 128, "kv_heads": max(1, width // 512), "dim": 128, "vdim": 128, "scale": 128 ** -0.5,
+                     "mask": {"size": 512, "pool": 64},
+                     "rot": {"base": 500000.0, "dims": 64, "scaling": {"factor": 8.0, "original": 4096, "fast": 32.0, "slow": 1.0}}}}
+    mam = {"type": "mamba2", "mixer": {"heads": 2 * width // 64, "vdim": 64, "state": 128, "groups": 8, "conv": 4, "norm_groups": 8}}
+    mls = {"type": "mlstm", "mixer": {"heads": width // 128, "dim": 128, "vdim": 128, "gate_cap": 15.0}}
+    dense = {"kind": "dense", "ff": {2048: 8192, 4096: 14336}.get(width, 3 * width), "limit": 7.0}
+    moe = {"kind": "moe", "expert": {"ff": width // 2}, "router": {"experts": 32, "top": 4, "scale": 2.5}, "shared": {"ff": width}}
+    pattern = [(att, dense), (mam, moe), (mls, dense), (mls, moe)]
+    raw = {"architecture": "Sominex", "vocab": 128256, "width": width, "norm": {"eps": 1e-5}, "embedding": {"scale": 1.0},
+           "layers": [{**pattern[i % 4][0], "mlp": pattern[i % 4][1]} for i in range(layers)]}
+    return SominexConfig(raw, context_len=context_len)
+
+
 def llama_config(width: int, layers: int, context_len: int):
     """the layers of Llama-3.2-1B (width 2048) / Llama-3-8B (width 4096), `layers` of them"""
     from scratchpad_amd.model_runner import ModelConfig
-    cfg = {2048: ModelConfig.llama32_1b, 4096: ModelConfig.llama3_8b}[width](context_len)
+    if width in (2048, 4096):
+        cfg = {2048: ModelConfig.llama32_1b, 4096: ModelConfig.llama3_8b}[width](context_len)
+    else:          # the same proportions at another width: heads of 128, a quarter as many key/value heads, ff = 3.5 width
+        cfg = ModelConfig(width, 7 * width // 2, layers, width // 128, max(1, width // 512), 128256, context_len=context_len,
+                          head_dim=128)
     cfg.num_hidden_layers = layers
     return cfg
 
@@ -122,6 +144,31 @@ def instrument(clock: KernelClock, cfg):
         R = q_rot.shape[2]
         return _nbytes(q_lat, out) + clock.keys_read() * (C + R) * pool.element_size(), 2 * H * clock.pairs() * (2 * C + R), MATRIX
 
+    def window(a, k, out):
+        q, kpool, vpool = a[0], a[1], a[2]
+        H, G, D, Dv, size, P = a[7], a[8], a[9], a[10], a[11], a[12]
+        seen = 0                 # (query, visible key or block) pairs
+        for p, e in zip(clock.step["prefix"], clock.step["extend"]):
+            for pos in (range(p, p + e) if e <= 4 else ()):
+                seen += min(pos + 1, size) + (max(pos - size + 1, 0) // P if P else 0)
+            if e > 4:            # closed form for a long portion: the window term, then the block term
+                full = [min(pos + 1, size) for pos in (p, p + e - 1)]
+                seen += e * (full[0] + full[1]) // 2 + (sum(max(pos - size + 1, 0) // P for pos in range(p, p + e, 64)) * 64 if P else 0)
+        rows = sum(min(p + e, size + e) + ((p + e) // P if P else 0) for p, e in zip(clock.step["prefix"], clock.step["extend"]))
+        return _nbytes(q, out) + rows * G * (D + Dv) * kpool.element_size(), 2 * H * seen * (D + Dv), MATRIX
+
+    def scan(a, k, out):         # state in and out once per (request, head); 4 flops per state element and token
+        xbc, state, heads, N, Dv = a[0], a[5], a[7], a[9], a[10]
+        return _nbytes(xbc, out) + 2 * len(clock.step["extend"]) * heads * N * Dv * 4, 4 * xbc.shape[0] * heads * N * Dv, VECTOR32
+
+    def mlstm(a, k, out):
+        q, S, heads, D, Dv = a[0], a[7], a[11], a[12], a[13]
+        return _nbytes(*a[:4], out) + 2 * len(clock.step["extend"]) * heads * D * Dv * 4, 4 * q.shape[0] * heads * D * Dv, VECTOR32
+
+    def small(a, k, out):
+        x, w = a[0], a[1]
+        return _nbytes(x, w, out), 2 * x.shape[0] * w.shape[0] * w.shape[1], VECTOR32
+
     def llama_extend(a, k, out):
         o, q, kb = a[0], a[1], a[2]
         H, D, Hkv = q.shape[1], q.shape[2], kb.shape[1]
@@ -131,7 +178,10 @@ def instrument(clock: KernelClock, cfg):
              "token_shift": io, "wkv_decay": io, "wkv_recurrence": wkv, "rotary_interleaved": io, "latent_kv_store": io,
              "latent_attention": latent, "moe_route": io, "moe_align": io, "moe_grouped_gemm": grouped, "moe_glu": io,
              "moe_combine": io, "rmsnorm": io, "fused_add_rmsnorm": io, "silu_and_mul": io, "rotary_embedding": io,
-             "extend_attention": llama_extend, "decode_attention": llama_extend, "linear": gemm, "linear_silu_mul": gemm}
+             "extend_attention": llama_extend, "decode_attention": llama_extend, "linear": gemm, "linear_silu_mul": gemm,
+             "embed_scale": io, "norm_shift": io, "stream_add": io, "qkv_rotary_store": io, "pool_blocks": io,
+             "window_attention": window, "small_linear_f32": small, "causal_conv_silu": io, "mamba2_scan": scan,
+             "gated_group_norm": io, "mlstm_scan": mlstm, "moe_route_softmax": io}
     for name, cost in costs.items():
         saved[name] = getattr(N, name)
         setattr(N, name, clock.record(name, saved[name], cost))
@@ -238,10 +288,11 @@ DISABLED = ("bench.py --mode hybrid is switched off: its whole-model pass at the
             "(tests/test_gpu_tizalorn_kernels.py).  It stays off the GPU until the cause is shown.")
 
 
-def hybrid_main(args):
+def hybrid_main(args, design: str = "tizalorn"):
     """the parent: never touches the GPU; one child process per (model, size), so that neither model's graphs, pools or
     library workspaces are in the other's process"""
-    raise SystemExit(DISABLED)
+    if design == "tizalorn":
+        raise SystemExit(DISABLED)
     import argparse
     import os
     import subprocess
@@ -258,7 +309,7 @@ def hybrid_main(args):
     runs = []
     for w in widths:
         row = {"width": w, "layers": layers}
-        for model in ("tizalorn", "llama"):
+        for model in (design, "llama"):
             cmd = [sys.executable, "-u", os.path.abspath(__file__), "--child", model, "--width", str(w), "--layers", str(layers),
                    "--bs", str(args.bs), "--ctx", str(args.ctx), "--steps", str(args.steps), "--warmup", str(args.warmup),
                    "--max-prefill-tokens", str(args.max_prefill_tokens)]
@@ -275,31 +326,32 @@ def hybrid_main(args):
         runs.append(row)
     last = runs[-1]
     print(json.dumps({
-        "metric": "hybrid_decode_tokens_per_sec", "value": last["tizalorn"]["decode_tokens_per_sec"], "unit": "tokens/s",
-        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": last["tizalorn"]["decode_ms_per_step"],
+        "metric": f"{design}_decode_tokens_per_sec", "value": last[design]["decode_tokens_per_sec"], "unit": "tokens/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": last[design]["decode_ms_per_step"],
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
         "data": "synthetic (random-init weights, random prompts)",
-        "config": {"workload": f"Tizalorn vs Llama layers at equal width and depth, bs={args.bs} prompts of {args.ctx} tokens, "
+        "config": {"workload": f"{design.capitalize()} vs Llama layers at equal width and depth, bs={args.bs} prompts of {args.ctx} tokens, "
                                f"extend batches <= {args.max_prefill_tokens} tokens, then {args.steps} decode steps, "
                                f"{'eager' if args.no_graph else 'HIP-graph replay'}", "sizes": runs}}), flush=True)
 
 
 def child_main():
-    raise SystemExit(DISABLED)
     import argparse
     import os
     import sys
     sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
     ap = argparse.ArgumentParser()
-    ap.add_argument("--child", required=True, choices=["tizalorn", "llama"])
+    ap.add_argument("--child", required=True, choices=["tizalorn", "sominex", "llama"])
     for name in ("width", "layers", "bs", "ctx", "steps", "warmup", "max-prefill-tokens"):
         ap.add_argument("--" + name, type=int, required=True)
     ap.add_argument("--no-graph", action="store_true")
     ap.add_argument("--no-kernel-table", action="store_true")
     a = ap.parse_args()
+    if a.child == "tizalorn":
+        raise SystemExit(DISABLED)
     torch.cuda.set_device(0)
     ctx_len = a.ctx + 2 * (a.steps + a.warmup) + 16
-    cfg = (tizalorn_config if a.child == "tizalorn" else llama_config)(a.width, a.layers, ctx_len)
+    cfg = {"sominex": sominex_config, "llama": llama_config}[a.child](a.width, a.layers, ctx_len)
     out = run_model(cfg, a, not a.no_kernel_table)
     print("RESULT " + json.dumps(out), flush=True)
 

@@ -481,10 +481,11 @@ SP_API int sp_moe_glu(void* out, const void* gu, int64_t pairs, int ff, float li
 SP_API int sp_moe_combine(void* out, const void* z, const int32_t* place, const float* weights, int64_t num_tokens,
                           int width, int top, int64_t out_stride, int dtype, void* stream);
 
-/* Router with softmax scores: z = router x in fp32, s = softmax(z) over all experts; ids [T, top] = the experts with the
- * largest s (ties: the lower index), weights [T, top] = their s times scale, not renormalised.                      */
-SP_API int sp_moe_route_softmax(int32_t* ids, float* weights, const void* x, int64_t x_stride, const float* router,
-                                int64_t num_tokens, int width, int experts, int top, float scale, int dtype, void* stream);
+/* Choice of experts by softmax scores on ready fp32 logits [T, experts] (sp_small_linear_f32 makes them): s = softmax
+ * over all experts; ids [T, top] = the experts with the largest s (ties: the lower index), weights [T, top] = their s
+ * times scale, not renormalised.                                                                                    */
+SP_API int sp_moe_softmax_topk(int32_t* ids, float* weights, const float* logits, int64_t num_tokens, int experts, int top,
+                               float scale, void* stream);
 
 /* ---- fp32 residual stream of parallel-sublayer layers (csrc/stream_norm.hip) ------------------------------------- */
 /* x[t] = embed[ids[t]] * scale  (x fp32, embed in `dtype`) */

@@ -125,7 +125,7 @@ SIGNATURES = {
     "sp_moe_glu": (_i32, [_vp, _vp, _i64, _i32, _f32, _f32, _i32, _vp]),
     "sp_moe_combine": (_i32, [_vp, _vp, _vp, _vp, _i64, _i32, _i32, _i64, _i32, _vp]),
     # ---- ABI 11
-    "sp_moe_route_softmax": (_i32, [_vp, _vp, _vp, _i64, _vp, _i64, _i32, _i32, _i32, _f32, _i32, _vp]),
+    "sp_moe_softmax_topk": (_i32, [_vp, _vp, _vp, _i64, _i32, _i32, _f32, _vp]),
     "sp_embed_scale": (_i32, [_vp, _i64, _vp, _vp, _i64, _i32, _i64, _f32, _i32, _vp]),
     "sp_norm_shift": (_i32, [_vp, _vp, _i64, _vp, _i64, _vp, _vp, _vp, _i64, _i64, _i32, _f32, *_SEQ, _i32, _vp]),
     "sp_norm_save_last": (_i32, [_vp, _i64, _vp, _i64, _vp, _i32, _f32, *_SEQ, _vp]),
@@ -1193,15 +1193,13 @@ def moe_combine(z: torch.Tensor, place: torch.Tensor, weights: torch.Tensor) -> 
 
 # --------------------------------------------------------------------------- fp32 stream with token shift, windowed attention, scans
 def moe_route_softmax(x: torch.Tensor, router: torch.Tensor, top: int, scale: float):
-    """(ids int32 [T, top], weights fp32 [T, top]): the largest softmax scores, times scale"""
-    _mat(x, "x"), _f32(router, "router")
-    T, E = x.shape[0], router.shape[0]
-    if router.shape[1] != x.shape[1]:
-        raise RuntimeError("moe_route_softmax: router [experts, width]")
+    """(ids int32 [T, top], weights fp32 [T, top]): fp32 logits router x, the largest softmax scores, times scale"""
+    logits = small_linear_f32(x, router)
+    T, E = logits.shape
     ids = torch.empty((T, top), dtype=torch.int32, device=x.device)
     weights = torch.empty((T, top), dtype=torch.float32, device=x.device)
-    _check(load().sp_moe_route_softmax(ids.data_ptr(), weights.data_ptr(), x.data_ptr(), x.stride(0), router.data_ptr(), T,
-                                       x.shape[1], E, top, scale, _dt(x), _stream()), "sp_moe_route_softmax")
+    _check(load().sp_moe_softmax_topk(ids.data_ptr(), weights.data_ptr(), logits.data_ptr(), T, E, top, scale, _stream()),
+           "sp_moe_softmax_topk")
     return ids, weights
 
 

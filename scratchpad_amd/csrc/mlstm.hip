@@ -5,54 +5,75 @@
 //   S' = exp(f + m - m') S + exp(i - m') k v^T          n' = exp(f + m - m') n + exp(i - m') k
 //   o  = S'^T q / (max(|n' . q|, exp(-m')) + 1e-6)      q = (projection) * D^(-1/2)
 //   out = o / rms_head(o) * w * sigmoid(g)
-// S, n and m start at ZERO for a sequence (m too: not minus infinity).  One workgroup per (request, head): thread j owns
-// column j of S in registers; every wave keeps its own copy of n in LDS (all copies identical), so a token costs no
-// workgroup barrier; tokens are staged through LDS in passes and the per-head norm and gate run as the pass's epilogue.
+// S, n and m start at ZERO for a sequence (m too: not minus infinity).  One workgroup per (request, head): a column of S
+// lives in the registers of 1, 2 or 4 neighbouring lanes; every wave keeps its own copy of n in LDS (all copies identical),
+// so a token costs no workgroup barrier; tokens are staged through LDS in passes and the per-head norm and gate run as the pass's epilogue.
 #include "seq_batch.h"
 
 namespace sp {
 namespace {
 
-constexpr int kChunk = 8;
+// tokens staged in LDS per pass (fewer for the widest heads: static + dynamic LDS stay under 64 KB)
+constexpr int chunk_of(int DP) { return DP > 128 ? 8 : 16; }
+// lanes that share one column of S: each holds at most 64 of the column's D values, so the state never crowds the
+// register file (at 128 values per lane the compiler is at its 256-register limit with one wave per SIMD, and every LDS
+// read of k and q waits in full)
+constexpr int split_of(int DP) { return DP > 128 ? 4 : (DP > 64 ? 2 : 1); }
 
 __device__ __forceinline__ float logsigmoid_f(float z) { return fminf(z, 0.f) - log1pf(expf(-fabsf(z))); }
 
+// thread = (column col of S, part): part p of SP owns the rows [p DS, (p + 1) DS) of the column; the parts of a column
+// are neighbouring lanes and add their partial numerators by lane exchange.  LDS rows of q and k are padded by 4 floats
+// per part so that the parts' simultaneous broadcast reads fall into different banks.
 template <typename Tag, int DP>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(256 * split_of(DP))
 mlstm_scan_kernel(void* out, int64_t out_stride, const void* q, int64_t q_stride, const void* k, int64_t k_stride,
                   const void* v, int64_t v_stride, const void* g, int64_t g_stride, const float* ipre, const float* fpre,
                   const float* norm_w, float* S_state, int64_t S_stride, float* n_state, int64_t n_stride, float* m_state,
                   int64_t m_stride, SeqBatch s, int H, int D, int Dv, float cap, float eps) {
   typedef Elem<Tag> E;
-  __shared__ float sq[kChunk][DP], sk[kChunk][DP], si[kChunk], sf[kChunk], sn[4][DP];
-  extern __shared__ float so[];                         // [kChunk][Dv]
+  constexpr int kChunk = chunk_of(DP), SP = split_of(DP), DS = DP / SP, ROW = DP + 4 * SP;
+  __shared__ float sq[kChunk][ROW], sk[kChunk][ROW], si[kChunk], sf[kChunk], sinv[kChunk], sn[4 * SP][DP];
+  extern __shared__ float so[];                         // [kChunk][Dv] outputs, then [kChunk][Dv] values
+  float* sv = so + (size_t)kChunk * Dv;                 // (no global load inside the token loop)
   const int b = blockIdx.x, h = blockIdx.y, j = threadIdx.x;
   const int nthreads = blockDim.x, wave = j >> 6, lane = j & 63, waves = nthreads >> 6;
+  const int col = j / SP, part = j % SP;
   int64_t start, len, prefix;
   seq_span(s, b, start, len, prefix);
   if (len <= 0) return;
-  const bool live = j < Dv;
+  const bool live = col < Dv;
   const int64_t slot = load_idx(s.req_pool_indices, b, s.idx64);
   float* Sst = S_state + slot * S_stride + (int64_t)h * D * Dv;
   float* nst = n_state + slot * n_stride + (int64_t)h * D;
   float* mst = m_state + slot * m_stride + h;
   const bool held = prefix > 0;
-  float S[DP];
+  float S[DS];
 #pragma unroll
-  for (int i = 0; i < DP; ++i) S[i] = (live && i < D && held) ? Sst[(int64_t)i * Dv + j] : 0.f;
+  for (int ii = 0; ii < DS; ++ii) {
+    const int i = part * DS + ii;
+    S[ii] = (live && i < D && held) ? Sst[(int64_t)i * Dv + col] : 0.f;
+  }
   for (int i = lane; i < DP; i += 64) sn[wave][i] = (i < D && held) ? nst[i] : 0.f;
   float m = held ? mst[0] : 0.f;
   const float qscale = 1.f / sqrtf((float)D);
   const int64_t colk = (int64_t)h * D, colv = (int64_t)h * Dv;
+  const float* myq = &sq[0][part * (DS + 4)];
+  const float* myk = &sk[0][part * (DS + 4)];
   for (int64_t c0 = 0; c0 < len; c0 += kChunk) {
     const int n = (int)(len - c0 < kChunk ? len - c0 : kChunk);
     __syncthreads();
-    for (int e = j; e < n * DP; e += nthreads) {
-      const int tt = e / DP, i = e % DP;
-      const int64_t row = start + c0 + tt;
-      const bool ok = i < D;
-      sq[tt][i] = ok ? E::load(q, row * q_stride + colk + i) * qscale : 0.f;
-      sk[tt][i] = ok ? E::load(k, row * k_stride + colk + i) : 0.f;
+    // staging: every load of the pass is issued before the first is used (rows past the pass's end repeat its last row)
+#pragma unroll
+    for (int tt = 0; tt < kChunk; ++tt) {
+      const int64_t row = start + c0 + (tt < n ? tt : n - 1);
+      for (int i = j; i < DP; i += nthreads) {
+        const bool ok = i < D;
+        const int at = i + 4 * (i / DS);
+        sq[tt][at] = ok ? E::load(q, row * q_stride + colk + i) * qscale : 0.f;
+        sk[tt][at] = ok ? E::load(k, row * k_stride + colk + i) : 0.f;
+      }
+      for (int c = j; c < Dv; c += nthreads) sv[tt * Dv + c] = E::load(v, row * v_stride + colv + c);
     }
     if (j < n) {
       const int64_t row = start + c0 + j;
@@ -61,45 +82,63 @@ mlstm_scan_kernel(void* out, int64_t out_stride, const void* q, int64_t q_stride
     }
     __syncthreads();
     for (int tt = 0; tt < n; ++tt) {
-      const int64_t row = start + c0 + tt;
       const float ig = si[tt], fg = sf[tt];
       const float m_new = fmaxf(fg + m, ig);
       const float keep = expf(fg + m - m_new), take = expf(ig - m_new);
       m = m_new;
       // this wave's copy of n, then n . q
-      float part = 0.f;
+      float dot = 0.f;
       for (int i = lane; i < DP; i += 64) {
-        const float nv = keep * sn[wave][i] + take * sk[tt][i];
+        const int at = i + 4 * (i / DS);
+        const float nv = keep * sn[wave][i] + take * sk[tt][at];
         sn[wave][i] = nv;
-        part += nv * sq[tt][i];
+        dot += nv * sq[tt][at];
       }
-      const float dot = wave_sum(part);
-      const float tv = take * (live ? E::load(v, row * v_stride + colv + j) : 0.f);
+      dot = wave_sum(dot);
+      const float tv = take * (live ? sv[tt * Dv + col] : 0.f);
+      const float* kq = myk + tt * ROW;
+      const float* qq = myq + tt * ROW;
       float num = 0.f;
 #pragma unroll
-      for (int i = 0; i < DP; ++i) {
-        S[i] = keep * S[i] + sk[tt][i] * tv;
-        num += S[i] * sq[tt][i];
+      for (int ii = 0; ii < DS; ++ii) {
+        S[ii] = keep * S[ii] + kq[ii] * tv;
+        num += S[ii] * qq[ii];
       }
-      if (live) so[tt * Dv + j] = num / (fmaxf(fabsf(dot), expf(-m_new)) + 1e-6f);
+#pragma unroll
+      for (int off = 1; off < SP; off <<= 1) num += __shfl_xor(num, off, 64);
+      if (live && part == 0) so[tt * Dv + col] = num / (fmaxf(fabsf(dot), expf(-m_new)) + 1e-6f);
     }
     __syncthreads();
+    // per-head RMS of every token of the pass (a wave per token, LDS only), then every column of all tokens at once
     for (int tt = wave; tt < n; tt += waves) {
       float ss = 0.f;
       for (int i = lane; i < Dv; i += 64) ss += so[tt * Dv + i] * so[tt * Dv + i];
       ss = wave_sum(ss);
-      const float inv = 1.f / sqrtf(ss / (float)Dv + eps);
-      const int64_t row = start + c0 + tt;
-      for (int i = lane; i < Dv; i += 64) {
-        const float gv = E::load(g, row * g_stride + colv + i);
-        E::store(out, row * out_stride + colv + i, so[tt * Dv + i] * inv * norm_w[colv + i] / (1.f + expf(-gv)));
+      if (lane == 0) sinv[tt] = 1.f / sqrtf(ss / (float)Dv + eps);
+    }
+    __syncthreads();
+    if (live) {                                         // part p takes the tokens p, p + SP, ...
+      const float nw = norm_w[colv + col];
+      constexpr int PER = kChunk / SP;
+      float gv[PER];
+#pragma unroll
+      for (int u = 0; u < PER; ++u) {
+        const int tt = part + u * SP;
+        gv[u] = E::load(g, (start + c0 + (tt < n ? tt : n - 1)) * g_stride + colv + col);
+      }
+#pragma unroll
+      for (int u = 0; u < PER; ++u) {
+        const int tt = part + u * SP;
+        if (tt < n) E::store(out, (start + c0 + tt) * out_stride + colv + col, so[tt * Dv + col] * sinv[tt] * nw / (1.f + expf(-gv[u])));
       }
     }
   }
   if (live) {
 #pragma unroll
-    for (int i = 0; i < DP; ++i)
-      if (i < D) Sst[(int64_t)i * Dv + j] = S[i];
+    for (int ii = 0; ii < DS; ++ii) {
+      const int i = part * DS + ii;
+      if (i < D) Sst[(int64_t)i * Dv + col] = S[ii];
+    }
   }
   if (wave == 0) {
     for (int i = lane; i < D; i += 64) nst[i] = sn[0][i];
@@ -114,12 +153,11 @@ static int launch_mlstm(void* out, int64_t out_stride, const void* q, int64_t q_
                         float* m_state, int64_t m_stride, const SeqBatch& s, int H, int D, int Dv, float cap, float eps,
                         hipStream_t st) {
   const dim3 grid((unsigned)s.B, (unsigned)H);
-  const unsigned threads = (unsigned)((Dv + 63) / 64 * 64);
-  const size_t lds = (size_t)kChunk * Dv * sizeof(float);
 #define SP_MLSTM(DP)                                                                                                    \
-  mlstm_scan_kernel<Tag, DP><<<grid, threads, lds, st>>>(out, out_stride, q, q_stride, k, k_stride, v, v_stride, g, g_stride, \
-                                                         ipre, fpre, norm_w, S_state, S_stride, n_state, n_stride, m_state,  \
-                                                         m_stride, s, H, D, Dv, cap, eps)
+  mlstm_scan_kernel<Tag, DP><<<grid, (unsigned)((Dv * split_of(DP) + 63) / 64 * 64),                                    \
+                               2 * (size_t)chunk_of(DP) * Dv * sizeof(float), st>>>(                                    \
+      out, out_stride, q, q_stride, k, k_stride, v, v_stride, g, g_stride, ipre, fpre, norm_w, S_state, S_stride, n_state,  \
+      n_stride, m_state, m_stride, s, H, D, Dv, cap, eps)
   if (D <= 16) SP_MLSTM(16);
   else if (D <= 32) SP_MLSTM(32);
   else if (D <= 64) SP_MLSTM(64);

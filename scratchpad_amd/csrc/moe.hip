@@ -79,12 +79,10 @@ __global__ void moe_route_kernel(int32_t* ids, float* weights, const void* x, in
   }
 }
 
-// ---- router with softmax scores: one wave per token -----------------------------------------------------------------
-// z = W x (fp32), s = softmax(z) over all experts; the `top` largest s win (ties: the lower index); weights = s * scale
-template <typename Tag>
-__global__ void moe_route_softmax_kernel(int32_t* ids, float* weights, const void* x, int64_t x_stride, const float* router,
-                                         int64_t T, int width, int E, int top, float scale) {
-  typedef Elem<Tag> El;
+// ---- softmax scores and choice on ready fp32 logits: one wave per token ---------------------------------------------
+// s = softmax(z) over all experts; the `top` largest s win (ties: the lower index); weights = s * scale
+__global__ void moe_softmax_topk_kernel(int32_t* ids, float* weights, const float* logits, int64_t T, int E, int top,
+                                        float scale) {
   extern __shared__ float smem[];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int64_t t = (int64_t)blockIdx.x * (blockDim.x >> 6) + wave;
@@ -92,19 +90,14 @@ __global__ void moe_route_softmax_kernel(int32_t* ids, float* weights, const voi
   float* score = smem + (size_t)wave * 2 * E;     // s[E], then the choice copy
   float* choice = score + E;
   float zmax = -INFINITY;
-  for (int e = 0; e < E; ++e) {
-    float d = 0.f;
-    for (int i = lane; i < width; i += 64) d += router[(int64_t)e * width + i] * El::load(x, t * x_stride + i);
-    d = wave_sum(d);
-    zmax = fmaxf(zmax, d);
-    if (lane == 0) score[e] = d;
-  }
-  __builtin_amdgcn_wave_barrier();
+  for (int e = lane; e < E; e += 64) zmax = fmaxf(zmax, logits[t * E + e]);
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) zmax = fmaxf(zmax, __shfl_xor(zmax, off, 64));
   float part = 0.f;
-  for (int e = lane; e < E; e += 64) part += expf(score[e] - zmax);
+  for (int e = lane; e < E; e += 64) part += expf(logits[t * E + e] - zmax);
   const float inv = 1.f / wave_sum(part);
   for (int e = lane; e < E; e += 64) {
-    const float sv = expf(score[e] - zmax) * inv;
+    const float sv = expf(logits[t * E + e] - zmax) * inv;
     score[e] = sv;
     choice[e] = sv;
   }
@@ -365,16 +358,15 @@ extern "C" int sp_moe_route(int32_t* ids, float* weights, const void* x, int64_t
   return SP_OK;
 }
 
-extern "C" int sp_moe_route_softmax(int32_t* ids, float* weights, const void* x, int64_t x_stride, const float* router,
-                                    int64_t num_tokens, int width, int experts, int top, float scale, int dtype,
-                                    void* stream) {
-  SP_CHECK_ARG(num_tokens >= 0 && width > 0 && experts > 0 && top > 0 && top <= experts);
+extern "C" int sp_moe_softmax_topk(int32_t* ids, float* weights, const float* logits, int64_t num_tokens, int experts, int top,
+                                   float scale, void* stream) {
+  SP_CHECK_ARG(num_tokens >= 0 && experts > 0 && top > 0 && top <= experts);
   if (num_tokens == 0) return SP_OK;
-  SP_CHECK_ARG(ids && weights && x && router && x_stride >= width);
+  SP_CHECK_ARG(ids && weights && logits);
   const size_t lds = 4 * (size_t)(2 * experts) * sizeof(float);
   if (lds > 64 * 1024) return SP_ERR_UNSUPPORTED;
-  SP_DISPATCH_DTYPE(dtype, (moe_route_softmax_kernel<Tag><<<dim3((unsigned)((num_tokens + 3) / 4)), 256, lds, (hipStream_t)stream>>>(
-                               ids, weights, x, x_stride, router, num_tokens, width, experts, top, scale)));
+  moe_softmax_topk_kernel<<<dim3((unsigned)((num_tokens + 3) / 4)), 256, lds, (hipStream_t)stream>>>(ids, weights, logits,
+                                                                                                  num_tokens, experts, top, scale);
   SP_LAUNCH_CHECK();
   return SP_OK;
 }

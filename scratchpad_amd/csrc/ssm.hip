@@ -14,19 +14,32 @@ namespace {
 
 __device__ __forceinline__ float softplus_f(float z) { return fmaxf(z, 0.f) + log1pf(expf(-fabsf(z))); }
 
-// one wave per token, all outputs in turn
+// one workgroup per (token, 16 outputs): every wave forms 4 outputs at once, so the loads of 4 weight rows are in flight
+// together and the token's row is read once per wave
 template <typename Tag>
 __global__ void __launch_bounds__(256)
 small_linear_f32_kernel(float* out, const void* x, int64_t x_stride, const float* w, const float* bias, int64_t T, int K, int N) {
   typedef Elem<Tag> E;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  const int64_t t = (int64_t)blockIdx.x * 4 + wave;
-  if (t >= T) return;
-  for (int n = 0; n < N; ++n) {
-    float d = 0.f;
-    for (int i = lane; i < K; i += 64) d += w[(int64_t)n * K + i] * E::load(x, t * x_stride + i);
-    d = wave_sum(d);
-    if (lane == 0) out[t * N + n] = d + (bias ? bias[n] : 0.f);
+  const int64_t t = blockIdx.x;
+  const int n0 = (blockIdx.y * 4 + wave) * 4;
+  if (n0 >= N) return;
+  const float* w0 = w + (int64_t)n0 * K;
+  const bool h1 = n0 + 1 < N, h2 = n0 + 2 < N, h3 = n0 + 3 < N;
+  float d0 = 0.f, d1 = 0.f, d2 = 0.f, d3 = 0.f;
+  for (int i = lane; i < K; i += 64) {
+    const float xv = E::load(x, t * x_stride + i);
+    d0 += w0[i] * xv;
+    if (h1) d1 += w0[K + i] * xv;
+    if (h2) d2 += w0[2 * (int64_t)K + i] * xv;
+    if (h3) d3 += w0[3 * (int64_t)K + i] * xv;
+  }
+  d0 = wave_sum(d0), d1 = wave_sum(d1), d2 = wave_sum(d2), d3 = wave_sum(d3);
+  if (lane == 0) {
+    out[t * N + n0] = d0 + (bias ? bias[n0] : 0.f);
+    if (h1) out[t * N + n0 + 1] = d1 + (bias ? bias[n0 + 1] : 0.f);
+    if (h2) out[t * N + n0 + 2] = d2 + (bias ? bias[n0 + 2] : 0.f);
+    if (h3) out[t * N + n0 + 3] = d3 + (bias ? bias[n0 + 3] : 0.f);
   }
 }
 
@@ -83,39 +96,57 @@ conv_state_kernel(float* state, int64_t state_stride, const void* in, int64_t in
   for (int k = 0; k < keep; ++k) st[(int64_t)k * C + c] = fresh[k];
 }
 
-constexpr int kChunk = 8;       // tokens staged in LDS per pass
+constexpr int kChunk = 16;      // tokens staged in LDS per pass
+// lanes that share one column of S: each holds at most 64 of the column's N values (at 128 per lane the state alone
+// fills the register file, one wave per SIMD remains and every LDS read of B and C waits in full)
+constexpr int split_of(int NP) { return NP > 128 ? 4 : (NP > 64 ? 2 : 1); }
 
-// one workgroup per (request, head); thread j owns column j of S (N values in registers)
+// one workgroup per (request, head); thread = (column col of S, part): part p of SP owns the rows [p NS, (p + 1) NS) of
+// the column, the parts are neighbouring lanes and add their partial outputs by lane exchange.  LDS rows of B and C are
+// padded by 4 floats per part so that the parts' simultaneous broadcast reads fall into different banks.
 template <typename Tag, int NP>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(256 * split_of(NP))
 mamba2_scan_kernel(float* y, int64_t y_stride, const void* xbc, int64_t xbc_stride, const float* dt_raw, const float* dt_bias,
                    const float* A_log, const float* Dskip, float* state, int64_t state_stride, SeqBatch s, int H, int G, int N,
                    int Dv) {
   typedef Elem<Tag> E;
-  __shared__ float sB[kChunk][NP], sC[kChunk][NP], sdt[kChunk], sdec[kChunk];
+  constexpr int SP = split_of(NP), NS = NP / SP, ROW = NP + 4 * SP;
+  __shared__ float sB[kChunk][ROW], sC[kChunk][ROW], sdt[kChunk], sdec[kChunk];
+  extern __shared__ float sx[];                         // [kChunk][Dv]: no global load inside the token loop
   const int b = blockIdx.x, h = blockIdx.y, j = threadIdx.x;
   const int nthreads = blockDim.x;
+  const int col = j / SP, part = j % SP;
   int64_t start, len, prefix;
   seq_span(s, b, start, len, prefix);
   if (len <= 0) return;
-  const bool live = j < Dv;
+  const bool live = col < Dv;
   const int g = h / (H / G);
   const int64_t inner = (int64_t)H * Dv;
   const int64_t colx = (int64_t)h * Dv, colB = inner + (int64_t)g * N, colC = inner + (int64_t)G * N + (int64_t)g * N;
   float* st = state + load_idx(s.req_pool_indices, b, s.idx64) * state_stride + (int64_t)h * N * Dv;
-  float S[NP];
+  float S[NS];
 #pragma unroll
-  for (int i = 0; i < NP; ++i) S[i] = (live && i < N && prefix > 0) ? st[(int64_t)i * Dv + j] : 0.f;
+  for (int ii = 0; ii < NS; ++ii) {
+    const int i = part * NS + ii;
+    S[ii] = (live && i < N && prefix > 0) ? st[(int64_t)i * Dv + col] : 0.f;
+  }
   const float a = expf(A_log[h]), bias = dt_bias[h], skip = Dskip[h];
+  const float* myB = &sB[0][part * (NS + 4)];
+  const float* myC = &sC[0][part * (NS + 4)];
   for (int64_t c0 = 0; c0 < len; c0 += kChunk) {
     const int n = (int)(len - c0 < kChunk ? len - c0 : kChunk);
     __syncthreads();
-    for (int e = j; e < n * NP; e += nthreads) {
-      const int tt = e / NP, i = e % NP;
-      const int64_t row = start + c0 + tt;
-      const bool ok = i < N;
-      sB[tt][i] = ok ? E::load(xbc, row * xbc_stride + colB + i) : 0.f;
-      sC[tt][i] = ok ? E::load(xbc, row * xbc_stride + colC + i) : 0.f;
+    // staging: every load of the pass is issued before the first is used (rows past the pass's end repeat its last row)
+#pragma unroll
+    for (int tt = 0; tt < kChunk; ++tt) {
+      const int64_t row = start + c0 + (tt < n ? tt : n - 1);
+      for (int i = j; i < NP; i += nthreads) {
+        const bool ok = i < N;
+        const int at = i + 4 * (i / NS);
+        sB[tt][at] = ok ? E::load(xbc, row * xbc_stride + colB + i) : 0.f;
+        sC[tt][at] = ok ? E::load(xbc, row * xbc_stride + colC + i) : 0.f;
+      }
+      for (int c = j; c < Dv; c += nthreads) sx[tt * Dv + c] = E::load(xbc, row * xbc_stride + colx + c);
     }
     if (j < n) {
       const float dt = softplus_f(dt_raw[(start + c0 + j) * H + h] + bias);
@@ -125,21 +156,27 @@ mamba2_scan_kernel(float* y, int64_t y_stride, const void* xbc, int64_t xbc_stri
     __syncthreads();
     for (int tt = 0; tt < n; ++tt) {
       const int64_t row = start + c0 + tt;
-      const float xj = live ? E::load(xbc, row * xbc_stride + colx + j) : 0.f;
+      const float xj = live ? sx[tt * Dv + col] : 0.f;
       const float dec = sdec[tt], dx = sdt[tt] * xj;
+      const float* Bt = myB + tt * ROW;
+      const float* Ct = myC + tt * ROW;
       float o = 0.f;
 #pragma unroll
-      for (int i = 0; i < NP; ++i) {
-        S[i] = dec * S[i] + sB[tt][i] * dx;
-        o += S[i] * sC[tt][i];
+      for (int ii = 0; ii < NS; ++ii) {
+        S[ii] = dec * S[ii] + Bt[ii] * dx;
+        o += S[ii] * Ct[ii];
       }
-      if (live) y[row * y_stride + colx + j] = o + skip * xj;
+#pragma unroll
+      for (int off = 1; off < SP; off <<= 1) o += __shfl_xor(o, off, 64);
+      if (live && part == 0) y[row * y_stride + colx + col] = o + skip * xj;
     }
   }
   if (live) {
 #pragma unroll
-    for (int i = 0; i < NP; ++i)
-      if (i < N) st[(int64_t)i * Dv + j] = S[i];
+    for (int ii = 0; ii < NS; ++ii) {
+      const int i = part * NS + ii;
+      if (i < N) st[(int64_t)i * Dv + col] = S[ii];
+    }
   }
 }
 
@@ -178,7 +215,8 @@ extern "C" int sp_small_linear_f32(float* out, const void* x, int64_t x_stride, 
   SP_CHECK_ARG(num_tokens >= 0 && k > 0 && n > 0);
   if (num_tokens == 0) return SP_OK;
   SP_CHECK_ARG(out && x && weight && x_stride >= k);
-  SP_DISPATCH_DTYPE(dtype, (small_linear_f32_kernel<Tag><<<dim3((unsigned)((num_tokens + 3) / 4)), 256, 0, (hipStream_t)stream>>>(
+  const dim3 grid((unsigned)num_tokens, (unsigned)((n + 15) / 16));
+  SP_DISPATCH_DTYPE(dtype, (small_linear_f32_kernel<Tag><<<grid, 256, 0, (hipStream_t)stream>>>(
                                out, x, x_stride, weight, bias, num_tokens, k, n)));
   SP_LAUNCH_CHECK();
   return SP_OK;
@@ -212,9 +250,8 @@ static int launch_mamba2(float* y, int64_t y_stride, const void* xbc, int64_t xb
                          const float* dt_bias, const float* A_log, const float* Dskip, float* state, int64_t state_stride,
                          const SeqBatch& s, int H, int G, int N, int Dv, hipStream_t st) {
   const dim3 grid((unsigned)s.B, (unsigned)H);
-  const unsigned threads = (unsigned)((Dv + 63) / 64 * 64);
 #define SP_SCAN(NP)                                                                                                    \
-  mamba2_scan_kernel<Tag, NP><<<grid, threads, 0, st>>>(y, y_stride, xbc, xbc_stride, dt_raw, dt_bias, A_log, Dskip, state, \
+  mamba2_scan_kernel<Tag, NP><<<grid, (unsigned)((Dv * split_of(NP) + 63) / 64 * 64), (size_t)kChunk * Dv * sizeof(float), st>>>(y, y_stride, xbc, xbc_stride, dt_raw, dt_bias, A_log, Dskip, state, \
                                                         state_stride, s, H, G, N, Dv)
   if (N <= 16) SP_SCAN(16);
   else if (N <= 32) SP_SCAN(32);

@@ -112,8 +112,10 @@ __device__ __forceinline__ float dot_row(const float* sq, const void* base, int6
   return d;
 }
 
-// One wave per (token, query head), 4 heads of a token per workgroup.  The query's keys are numbered blocks first, then
-// the window's tokens; tiles of 64: lane = key for the scores, lane = value channel for the weighted sum.
+// One workgroup of 4 waves per (token, query head).  The query's keys are numbered blocks first, then the window's
+// tokens, in tiles of 64; wave w takes tiles w, w + 4, ...: lane = key for the scores, lane = value channel for the
+// weighted sum (4 keys' rows in flight at a time); the waves' partial (maximum, sum, weighted values) meet in LDS.
+// The order of every sum depends on the query's position only, never on the batch or on how the prompt was cut.
 template <typename Tag, bool VEC>
 __global__ void __launch_bounds__(256)
 window_attention_kernel(void* out, int64_t out_stride, const void* q, int64_t q_stride, const void* kpool, const void* vpool,
@@ -124,10 +126,11 @@ window_attention_kernel(void* out, int64_t out_stride, const void* q, int64_t q_
   extern __shared__ float smem[];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int64_t t = blockIdx.x;
-  const int h = blockIdx.y * 4 + wave;
-  if (h >= H) return;                                    // (no workgroup barrier below)
-  float* sq = smem + (size_t)wave * (D + 64);
-  float* sw = sq + D;
+  const int h = blockIdx.y;
+  float* sq = smem;                              // [D] the scaled query
+  float* sw = smem + D + wave * 64;              // this wave's 64 weights
+  float* sacc = smem + D + 256;                  // [4][Dv]
+  float* sml = sacc + 4 * Dv;                    // [4] maxima, [4] sums
   int b;
   int64_t start, prefix;
   seq_of_token(s, t, b, start, prefix);
@@ -137,13 +140,14 @@ window_attention_kernel(void* out, int64_t out_stride, const void* q, int64_t q_
   const int64_t total = nb + (pos - w0 + 1);
   const int g = h / (H / G);
   const int32_t* table = req_to_token + load_idx(s.req_pool_indices, b, s.idx64) * table_stride;
-  for (int i = lane; i < D; i += 64) sq[i] = E::load(q, t * q_stride + (int64_t)h * D + i) * scale;
-  __builtin_amdgcn_wave_barrier();
+  for (int i = threadIdx.x; i < D; i += blockDim.x) sq[i] = E::load(q, t * q_stride + (int64_t)h * D + i) * scale;
+  __syncthreads();
   float m = -INFINITY, l = 0.f;
   float acc[kMaxPerLane];
 #pragma unroll
   for (int i = 0; i < kMaxPerLane; ++i) acc[i] = 0.f;
-  for (int64_t k0 = 0; k0 < total; k0 += 64) {
+  const int64_t vcol = (int64_t)g * Dv;
+  for (int64_t k0 = (int64_t)wave * 64; k0 < total; k0 += 256) {
     const int n = (int)(total - k0 < 64 ? total - k0 : 64);
     float sc = -INFINITY;
     if (lane < n) {
@@ -164,25 +168,66 @@ window_attention_kernel(void* out, int64_t out_stride, const void* q, int64_t q_
     __builtin_amdgcn_wave_barrier();
 #pragma unroll
     for (int i = 0; i < kMaxPerLane; ++i) acc[i] *= corr;
-    for (int j = 0; j < n; ++j) {
-      const int64_t kk = k0 + j;
-      const bool blk = kk < nb;
-      const int64_t row = blk ? table[kk * P + P - 1] : table[w0 + (kk - nb)];
-      const void* src = blk ? vpooled : vpool;
-      const float pj = sw[j];
+    int j = 0;
+    for (; j + 4 <= n; j += 4) {
+      int64_t at[4];
+      const void* src[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int64_t kk = k0 + j + u;
+        const bool blk = kk < nb;
+        at[u] = (int64_t)(blk ? table[kk * P + P - 1] : table[w0 + (kk - nb)]) * vp_stride + vcol;
+        src[u] = blk ? vpooled : vpool;
+      }
 #pragma unroll
       for (int i = 0; i < kMaxPerLane; ++i) {
         const int c = lane + 64 * i;
-        if (c < Dv) acc[i] += pj * E::load(src, row * vp_stride + (int64_t)g * Dv + c);
+        if (c < Dv) {
+          const float v0 = E::load(src[0], at[0] + c), v1 = E::load(src[1], at[1] + c);
+          const float v2 = E::load(src[2], at[2] + c), v3 = E::load(src[3], at[3] + c);
+          acc[i] += sw[j] * v0;
+          acc[i] += sw[j + 1] * v1;
+          acc[i] += sw[j + 2] * v2;
+          acc[i] += sw[j + 3] * v3;
+        }
+      }
+    }
+    for (; j < n; ++j) {
+      const int64_t kk = k0 + j;
+      const bool blk = kk < nb;
+      const int64_t at = (int64_t)(blk ? table[kk * P + P - 1] : table[w0 + (kk - nb)]) * vp_stride + vcol;
+      const void* src = blk ? vpooled : vpool;
+#pragma unroll
+      for (int i = 0; i < kMaxPerLane; ++i) {
+        const int c = lane + 64 * i;
+        if (c < Dv) acc[i] += sw[j] * E::load(src, at + c);
       }
     }
     __builtin_amdgcn_wave_barrier();
   }
-  const float inv = 1.f / l;
 #pragma unroll
   for (int i = 0; i < kMaxPerLane; ++i) {
     const int c = lane + 64 * i;
-    if (c < Dv) E::store(out, t * out_stride + (int64_t)h * Dv + c, acc[i] * inv);
+    if (c < Dv) sacc[wave * Dv + c] = acc[i];
+  }
+  if (lane == 0) {
+    sml[wave] = m;
+    sml[4 + wave] = l;
+  }
+  __syncthreads();
+  const float M = fmaxf(fmaxf(sml[0], sml[1]), fmaxf(sml[2], sml[3]));      // wave 0 always holds a key: M is finite
+  float e[4], den = 0.f;
+#pragma unroll
+  for (int w = 0; w < 4; ++w) {
+    e[w] = expf(sml[w] - M);                                               // a wave without keys: exp(-inf) = 0
+    den += sml[4 + w] * e[w];
+  }
+  const float inv = 1.f / den;
+  for (int c = threadIdx.x; c < Dv; c += blockDim.x) {
+    float num = 0.f;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) num += sacc[w * Dv + c] * e[w];
+    E::store(out, t * out_stride + (int64_t)h * Dv + c, num * inv);
   }
 }
 
@@ -240,10 +285,10 @@ extern "C" int sp_window_attention(void* out, int64_t out_stride, const void* q,
   SP_CHECK_ARG(q_stride >= (int64_t)heads * dim && out_stride >= (int64_t)heads * vdim);
   SP_CHECK_ARG(kp_stride >= (int64_t)kv_heads * dim && vp_stride >= (int64_t)kv_heads * vdim);
   if (vdim > 64 * kMaxPerLane) return SP_ERR_UNSUPPORTED;
-  const size_t lds = 4 * (size_t)(dim + 64) * sizeof(float);
+  const size_t lds = ((size_t)dim + 256 + 4 * (size_t)vdim + 8) * sizeof(float);
   if (lds > 64 * 1024) return SP_ERR_UNSUPPORTED;
   SEQ_BATCH(s);
-  const dim3 grid((unsigned)num_tokens, (unsigned)((heads + 3) / 4));
+  const dim3 grid((unsigned)num_tokens, (unsigned)heads);
   const int vecn = dtype == SP_F32 ? 4 : 8;
   const bool vec = dim % vecn == 0 && kp_stride % vecn == 0 && ((uintptr_t)kpool & 15) == 0 &&
                    (!kpooled || ((uintptr_t)kpooled & 15) == 0);
