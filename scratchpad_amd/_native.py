@@ -1301,11 +1301,17 @@ def window_attention(q: torch.Tensor, kpool: torch.Tensor, vpool: torch.Tensor, 
     return out
 
 
+SMALL_LINEAR_OWN_ROWS = 64      # up to this many rows small_linear_f32 runs on the library's own kernel
+
+
 def small_linear_f32(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
     """fp32 [T, n] = x @ weight.T + bias with fp32 weights, accumulation and output (gates and step sizes of recurrences)"""
     _mat(x, "x"), _f32(weight, "weight")
     if weight.dim() != 2 or weight.shape[1] != x.shape[1] or (bias is not None and _f32(bias, "bias").shape[0] != weight.shape[0]):
         raise RuntimeError("small_linear_f32: weight [n, k], bias [n]")
+    if x.shape[0] > SMALL_LINEAR_OWN_ROWS:
+        # many rows: the own kernel reads the weight rows again for every token; the library's fp32 product tiles them
+        return torch.nn.functional.linear(x.to(torch.float32), weight, bias)
     out = torch.empty((x.shape[0], weight.shape[0]), dtype=torch.float32, device=x.device)
     _check(load().sp_small_linear_f32(out.data_ptr(), x.data_ptr(), x.stride(0), weight.data_ptr(), _ptr(bias), x.shape[0],
                                       x.shape[1], weight.shape[0], _dt(x), _stream()), "sp_small_linear_f32")
