@@ -49,7 +49,9 @@ LAYERS = [
     (U.mamba2(4, 16, 24, groups=2, conv=4, norm_groups=2), None),
     (U.mamba2(3, 40, 8, groups=3, conv=2, norm_groups=1), None),              # a group per head
     (U.mamba2(1, 80, 72, groups=1, conv=5, norm_groups=5), None),
+    (U.mamba2(2, 136, 136, groups=2, conv=3, norm_groups=4), None),          # state and head width above 128
     (U.mlstm(3, 16, 24), None), (U.mlstm(1, 72, 8, cap=3.0), None), (U.mlstm(4, 8, 80), None),
+    (U.mlstm(2, 136, 136, cap=20.0), None), (U.attention(2, 1, 136, 200, size=33, pool=5, dims=72), None),
     (U.mlstm(2, 16, 16), U.dense(100)), (U.mlstm(2, 16, 16), U.dense(40, limit=0.3)),
     (U.mlstm(2, 16, 16), U.moe(12, 3, 24, scale=2.0, shared=56)), (U.mlstm(2, 16, 16), U.moe(5, 1, 40, scale=1.0)),
     (U.mlstm(2, 16, 16), U.moe(4, 4, 16, shared=8)),
