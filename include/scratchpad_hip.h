@@ -520,12 +520,13 @@ SP_API int sp_pool_blocks(void* kpooled, void* vpooled, const void* kpool, const
 /* out [T, heads, vdim]: a query at position p attends, in one fp32 softmax of (q . k) * scale, to the cached tokens j with
  * 0 <= p - j < window and to the pooled rows of the blocks b with b * block + block - 1 <= p - window.  window <= 0: every
  * earlier token and no blocks; block <= 0: no blocks.  Query head h reads key/value head h / (heads / kv_heads).
- * vdim <= 256.                                                                                                        */
+ * vdim <= 256.  matrix != 0: steps that bring portions of prompts in a 16-bit type, with dim and vdim of 64 or 128, run on
+ * the matrix cores (16 tokens x one key/value head per workgroup); everything else on the fp32 vector kernel.         */
 SP_API int sp_window_attention(void* out, int64_t out_stride, const void* q, int64_t q_stride, const void* kpool,
                                const void* vpool, const void* kpooled, const void* vpooled, int64_t kp_stride,
                                int64_t vp_stride, const int32_t* req_to_token, int64_t table_stride, int64_t num_tokens,
                                int heads, int kv_heads, int dim, int vdim, int64_t window, int block, float scale,
-                               SP_SEQ_PARAMS, int dtype, void* stream);
+                               int matrix, SP_SEQ_PARAMS, int dtype, void* stream);
 
 /* ---- state-space and matrix-memory recurrences (csrc/ssm.hip, csrc/mlstm.hip) -------------------------------------- */
 /* out[t, j] = bias[j] + sum_i weight[j, i] x[t, i]: fp32 weights, accumulation and output (x in `dtype`; bias optional) */

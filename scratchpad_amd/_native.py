@@ -134,7 +134,7 @@ SIGNATURES = {
                                    _i32, _i32, _i32, _i32, _f32, _i32, _vp]),
     "sp_pool_blocks": (_i32, [_vp, _vp, _vp, _vp, _i64, _i64, _vp, _i64, _i64, _i32, _i32, _i32, *_SEQ, _i32, _vp]),
     "sp_window_attention": (_i32, [_vp, _i64, _vp, _i64, _vp, _vp, _vp, _vp, _i64, _i64, _vp, _i64, _i64, _i32, _i32, _i32,
-                                   _i32, _i64, _i32, _f32, *_SEQ, _i32, _vp]),
+                                   _i32, _i64, _i32, _f32, _i32, *_SEQ, _i32, _vp]),
     "sp_small_linear_f32": (_i32, [_vp, _vp, _i64, _vp, _vp, _i64, _i32, _i32, _i32, _vp]),
     "sp_causal_conv_silu": (_i32, [_vp, _i64, _vp, _i64, _vp, _vp, _vp, _i64, _i64, _i32, _i32, *_SEQ, _i32, _vp]),
     "sp_mamba2_scan": (_i32, [_vp, _i64, _vp, _i64, _vp, _vp, _vp, _vp, _vp, _i64, _i32, _i32, _i32, _i32, *_SEQ, _i32, _vp]),
@@ -1284,8 +1284,9 @@ def pool_blocks(kpooled: torch.Tensor, vpooled: torch.Tensor, kpool: torch.Tenso
 
 def window_attention(q: torch.Tensor, kpool: torch.Tensor, vpool: torch.Tensor, kpooled: Optional[torch.Tensor],
                      vpooled: Optional[torch.Tensor], req_to_token: torch.Tensor, seq: SeqParams, heads: int, kv_heads: int,
-                     dim: int, vdim: int, window: int, block: int, scale: float) -> torch.Tensor:
-    """q [T, heads * dim] (rotated) -> [T, heads * vdim]"""
+                     dim: int, vdim: int, window: int, block: int, scale: float, matrix: bool = True) -> torch.Tensor:
+    """q [T, heads * dim] (rotated) -> [T, heads * vdim]; matrix=False keeps 16-bit prompt portions off the matrix-core
+    kernel (comparisons)"""
     _mat(q, "q"), _mat(kpool, "kpool"), _mat(vpool, "vpool")
     T = q.shape[0]
     if q.shape[1] != heads * dim or kpool.shape[1] != kv_heads * dim or vpool.shape[1] != kv_heads * vdim or \
@@ -1297,7 +1298,7 @@ def window_attention(q: torch.Tensor, kpool: torch.Tensor, vpool: torch.Tensor, 
     _check(load().sp_window_attention(out.data_ptr(), out.stride(0), q.data_ptr(), q.stride(0), kpool.data_ptr(),
                                       vpool.data_ptr(), _ptr(kpooled), _ptr(vpooled), kpool.stride(0), vpool.stride(0),
                                       req_to_token.data_ptr(), req_to_token.stride(0), T, heads, kv_heads, dim, vdim,
-                                      window, block, scale, *seq.args, _dt(q), _stream()), "sp_window_attention")
+                                      window, block, scale, int(matrix), *seq.args, _dt(q), _stream()), "sp_window_attention")
     return out
 
 

@@ -231,6 +231,191 @@ window_attention_kernel(void* out, int64_t out_stride, const void* q, int64_t q_
   }
 }
 
+
+// ---- the same attention on the matrix cores, for portions of prompts in 16-bit types ------------------------------------
+// One workgroup per (16 consecutive tokens of one request's portion, key/value head); wave w works for the group's query
+// head w (w + 4, ... in further passes).  Keys of the 16 queries' UNION (blocks up to the last query's, tokens from the
+// first query's window start to the last query) go by in tiles of 64; who sees what is a mask per (key, query).
+//   S^T = K Q^T   v_mfma_f32_16x16x32: first operand = 16 key rows straight from the pool (16 bytes per lane), second =
+//                 the query fragment held in registers; a lane receives S^T[key 4q + r][query r16]: four keys of ONE query,
+//                 so the softmax of a query is a reduction over r, the tile's four key groups and the lanes q = 0..3.
+//   O^T = V^T P^T first operand = V^T from an LDS tile written transposed ([value channel][key], keys contiguous), second =
+//                 P^T - exactly the registers the lane already holds: the key order inside a step of 32 is (4q .. 4q + 3 of
+//                 the first 16 keys, then of the second 16) for both operands, so P needs no exchange between lanes.
+// Scores, softmax and O are fp32; P enters the second product as a 16-bit value plus its 16-bit remainder (two products).
+typedef float f32x4_w __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8_w __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8_w __attribute__((ext_vector_type(8)));
+template <typename Tag>
+__device__ __forceinline__ f32x4_w mfma_w(const u32x4& a, const u32x4& b, const f32x4_w& c);
+template <>
+__device__ __forceinline__ f32x4_w mfma_w<bf16_tag>(const u32x4& a, const u32x4& b, const f32x4_w& c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_w, a), __builtin_bit_cast(bf16x8_w, b), c, 0, 0, 0);
+}
+template <>
+__device__ __forceinline__ f32x4_w mfma_w<f16_tag>(const u32x4& a, const u32x4& b, const f32x4_w& c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8_w, a), __builtin_bit_cast(f16x8_w, b), c, 0, 0, 0);
+}
+
+constexpr int kVtRow = 72;      // 64 keys + 8 of padding per value channel (16-bit elements)
+
+template <typename Tag, int DS, int DT>      // DS = dim / 32, DT = vdim / 16
+__global__ void __launch_bounds__(256)
+window_attention_mfma_kernel(void* out, int64_t out_stride, const void* q, int64_t q_stride, const void* kpool,
+                             const void* vpool, const void* kpooled, const void* vpooled, int64_t kp_stride, int64_t vp_stride,
+                             const int32_t* req_to_token, int64_t table_stride, SeqBatch s, int H, int G, int64_t size, int P,
+                             float scale) {
+  constexpr int D = 32 * DS, Dv = 16 * DT;
+  __shared__ uint16_t vt[Dv][kVtRow];
+  __shared__ int32_t sslot[64];
+  // which request and which of its 16-row tiles
+  int tile = blockIdx.x, b = 0;
+  for (; b < s.B; ++b) {
+    const int tiles = (s.extend_seq_lens[b] + 15) / 16;
+    if (tile < tiles) break;
+    tile -= tiles;
+  }
+  if (b >= s.B) return;
+  const int g = blockIdx.y, R = H / G;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, r16 = lane & 15, qd = lane >> 4;
+  const int64_t start = s.extend_start_loc[b], len = s.extend_seq_lens[b], prefix = s.extend_prefix_lens[b];
+  const int rows = (int)(len - 16 * tile < 16 ? len - 16 * tile : 16);
+  const int64_t t0 = start + 16 * tile, pos0 = prefix + 16 * tile, pos_last = pos0 + rows - 1;
+  const int32_t* table = req_to_token + load_idx(s.req_pool_indices, b, s.idx64) * table_stride;
+  const bool pooled = size > 0 && P > 0;
+  const int64_t w0U = (size > 0 && pos0 - size + 1 > 0) ? pos0 - size + 1 : 0;
+  const int64_t w0L = (size > 0 && pos_last - size + 1 > 0) ? pos_last - size + 1 : 0;
+  const int64_t nbU = pooled ? w0L / P : 0;
+  const int64_t totalU = nbU + (pos_last - w0U + 1);
+  // this lane's query (column r16 of every S^T tile)
+  const bool qvalid = r16 < rows;
+  const int64_t pos_q = pos0 + r16;
+  const int64_t w0_q = (size > 0 && pos_q - size + 1 > 0) ? pos_q - size + 1 : 0;
+  const int64_t nb_q = pooled ? w0_q / P : 0;
+  for (int h0 = 0; h0 < R; h0 += 4) {
+    const int hq = g * R + h0 + wave;
+    const bool work = h0 + wave < R;
+    u32x4 qf[DS];
+#pragma unroll
+    for (int st = 0; st < DS; ++st)
+      qf[st] = (work && qvalid) ? ld16((const char*)q + ((t0 + r16) * q_stride + (int64_t)hq * D + 32 * st + 8 * qd) * 2)
+                                : u32x4{0u, 0u, 0u, 0u};
+    f32x4_w oacc[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) oacc[dt] = f32x4_w{0.f, 0.f, 0.f, 0.f};
+    float m = -INFINITY, l = 0.f;
+    for (int64_t k0 = 0; k0 < totalU; k0 += 64) {
+      __syncthreads();                                   // the previous tile's readers are done
+      if (threadIdx.x < 64) {
+        const int64_t kk = k0 + threadIdx.x;
+        int32_t sl = 0;
+        if (kk < totalU) sl = kk < nbU ? table[kk * P + P - 1] : table[w0U + (kk - nbU)];
+        sslot[threadIdx.x] = sl;
+      }
+      __syncthreads();
+      // V^T tile: thread = (key, 8 value channels); neighbouring lanes take neighbouring keys (conflict-free 2-byte writes)
+      for (int c = threadIdx.x; c < 64 * (Dv / 8); c += 256) {
+        const int key = c & 63, dvc = c >> 6;
+        const int64_t kk = k0 + key;
+        u32x4 val = {0u, 0u, 0u, 0u};
+        if (kk < totalU)
+          val = ld16((const char*)(kk < nbU ? vpooled : vpool) + ((int64_t)sslot[key] * vp_stride + (int64_t)g * Dv + 8 * dvc) * 2);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const uint32_t w2 = e == 0 ? val[0] : (e == 1 ? val[1] : (e == 2 ? val[2] : val[3]));
+          vt[8 * dvc + 2 * e][key] = (uint16_t)(w2 & 0xffffu);
+          vt[8 * dvc + 2 * e + 1][key] = (uint16_t)(w2 >> 16);
+        }
+      }
+      __syncthreads();
+      if (work) {
+        f32x4_w sacc[4];
+#pragma unroll
+        for (int sb = 0; sb < 4; ++sb) {
+          sacc[sb] = f32x4_w{0.f, 0.f, 0.f, 0.f};
+          const int64_t kk = k0 + 16 * sb + r16;         // the key row this lane feeds
+          const bool kvalid = kk < totalU;
+          const char* kp = (const char*)(kk < nbU ? kpooled : kpool) + ((int64_t)sslot[16 * sb + r16] * kp_stride + (int64_t)g * D + 8 * qd) * 2;
+#pragma unroll
+          for (int st = 0; st < DS; ++st) {
+            const u32x4 a = kvalid ? ld16(kp + 64 * st) : u32x4{0u, 0u, 0u, 0u};
+            sacc[sb] = mfma_w<Tag>(a, qf[st], sacc[sb]);
+          }
+        }
+        float mx = -INFINITY;
+#pragma unroll
+        for (int sb = 0; sb < 4; ++sb)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const int64_t kk = k0 + 16 * sb + 4 * qd + r;
+            bool vis = qvalid && kk < totalU;
+            if (vis) {
+              if (kk < nbU) vis = kk < nb_q;
+              else {
+                const int64_t j = w0U + (kk - nbU);
+                vis = j >= w0_q && j <= pos_q;
+              }
+            }
+            const float v = vis ? sacc[sb][r] * scale : -INFINITY;
+            sacc[sb][r] = v;
+            mx = fmaxf(mx, v);
+          }
+        mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        const float m_new = fmaxf(m, mx);
+        const float m_safe = m_new == -INFINITY ? 0.f : m_new;      // nothing seen yet: every weight is exp(-inf) = 0
+        const float corr = expf(m - m_safe);
+        float psum = 0.f;
+        float pf[2][8];
+#pragma unroll
+        for (int sb = 0; sb < 4; ++sb)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const float p = expf(sacc[sb][r] - m_safe);
+            psum += p;
+            pf[sb >> 1][4 * (sb & 1) + r] = p;
+          }
+        psum += __shfl_xor(psum, 16, 64);
+        psum += __shfl_xor(psum, 32, 64);
+        l = l * corr + psum;
+        m = m_new;
+#pragma unroll
+        for (int hh = 0; hh < 2; ++hh) {
+          // the weights enter the product as a 16-bit value plus a 16-bit remainder: they are never rounded to 8 bits of
+          // mantissa (the second product costs an eighth of the step's matrix work again)
+          const u32x4 pb = pack16<Tag>(pf[hh]);
+          float rest[8], back[8];
+          unpack16<Tag>(pb, back);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) rest[e] = pf[hh][e] - back[e];
+          const u32x4 pr = pack16<Tag>(rest);
+#pragma unroll
+          for (int dt = 0; dt < DT; ++dt) {
+            if (hh == 0) {
+#pragma unroll
+              for (int r = 0; r < 4; ++r) oacc[dt][r] *= corr;
+            }
+            const u32x2 lo = *(const u32x2*)&vt[16 * dt + r16][32 * hh + 4 * qd];
+            const u32x2 hi = *(const u32x2*)&vt[16 * dt + r16][32 * hh + 16 + 4 * qd];
+            const u32x4 a = {lo[0], lo[1], hi[0], hi[1]};
+            oacc[dt] = mfma_w<Tag>(a, pb, oacc[dt]);
+            oacc[dt] = mfma_w<Tag>(a, pr, oacc[dt]);
+          }
+        }
+      }
+    }
+    if (work && qvalid) {
+      const float inv = 1.f / l;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) {
+        float f[8] = {oacc[dt][0] * inv, oacc[dt][1] * inv, oacc[dt][2] * inv, oacc[dt][3] * inv, 0.f, 0.f, 0.f, 0.f};
+        const u32x4 pk = pack16<Tag>(f);
+        *(u32x2*)((char*)out + ((t0 + r16) * out_stride + (int64_t)hq * Dv + 16 * dt + 4 * qd) * 2) = u32x2{pk[0], pk[1]};
+      }
+    }
+  }
+}
+
 }  // namespace
 }  // namespace sp
 
@@ -275,7 +460,7 @@ extern "C" int sp_window_attention(void* out, int64_t out_stride, const void* q,
                                    const void* vpool, const void* kpooled, const void* vpooled, int64_t kp_stride,
                                    int64_t vp_stride, const int32_t* req_to_token, int64_t table_stride,
                                    int64_t num_tokens, int heads, int kv_heads, int dim, int vdim, int64_t window, int block,
-                                   float scale, SP_SEQ_PARAMS, int dtype, void* stream) {
+                                   float scale, int matrix, SP_SEQ_PARAMS, int dtype, void* stream) {
   SP_CHECK_ARG(num_tokens >= 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0 && dim > 0 && vdim > 0);
   if (num_tokens == 0) return SP_OK;
   SP_CHECK_ARG(out && q && kpool && vpool && req_to_token && req_pool_indices && seq_lens);
@@ -288,6 +473,30 @@ extern "C" int sp_window_attention(void* out, int64_t out_stride, const void* q,
   const size_t lds = ((size_t)dim + 256 + 4 * (size_t)vdim + 8) * sizeof(float);
   if (lds > 64 * 1024) return SP_ERR_UNSUPPORTED;
   SEQ_BATCH(s);
+  // portions of prompts in 16-bit types: the matrix-core kernel where its tile shapes and 16-byte row loads apply
+  const bool al16 = (((uintptr_t)q | (uintptr_t)kpool | (uintptr_t)vpool | (uintptr_t)kpooled | (uintptr_t)vpooled) & 15) == 0 &&
+                    ((uintptr_t)out & 7) == 0;
+  if (matrix && extend_seq_lens && num_tokens > batch_size && (dtype == SP_BF16 || dtype == SP_F16) && (dim == 64 || dim == 128) &&
+      (vdim == 64 || vdim == 128) && al16 && q_stride % 8 == 0 && kp_stride % 8 == 0 && vp_stride % 8 == 0 && out_stride % 4 == 0) {
+    const dim3 mgrid((unsigned)((num_tokens + 15) / 16 + batch_size), (unsigned)kv_heads);
+#define SP_WM(T, DS, DT)                                                                                                 \
+  window_attention_mfma_kernel<T, DS, DT><<<mgrid, 256, 0, (hipStream_t)stream>>>(                                         \
+      out, out_stride, q, q_stride, kpool, vpool, kpooled, vpooled, kp_stride, vp_stride, req_to_token, table_stride, s, heads, \
+      kv_heads, window, block, scale)
+#define SP_WM_SHAPES(T)                                   \
+  do {                                                    \
+    if (dim == 64 && vdim == 64) SP_WM(T, 2, 4);          \
+    else if (dim == 64) SP_WM(T, 2, 8);                   \
+    else if (vdim == 64) SP_WM(T, 4, 4);                  \
+    else SP_WM(T, 4, 8);                                  \
+  } while (0)
+    if (dtype == SP_BF16) SP_WM_SHAPES(bf16_tag);
+    else SP_WM_SHAPES(f16_tag);
+#undef SP_WM_SHAPES
+#undef SP_WM
+    SP_LAUNCH_CHECK();
+    return SP_OK;
+  }
   const dim3 grid((unsigned)num_tokens, (unsigned)heads);
   const int vecn = dtype == SP_F32 ? 4 : 8;
   const bool vec = dim % vecn == 0 && kp_stride % vecn == 0 && ((uintptr_t)kpool & 15) == 0 &&

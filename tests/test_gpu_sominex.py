@@ -90,7 +90,7 @@ class AttnBench:
     """one request on row 2 of a request table whose slots are a shuffled part of a pool: the store, the block means and
     the attention kernel driven the way the model drives them, in portions"""
 
-    def __init__(self, H, G, D, Dv, size, P, rot=None, dtype=torch.float32, slots=400, seed=0):
+    def __init__(self, H, G, D, Dv, size, P, rot=None, dtype=torch.float32, slots=400, seed=0, matrix=True):
         from scratchpad_amd import _native
         from scratchpad_amd.layers import HalfAngleRotary
         self.n, self.H, self.G, self.D, self.Dv, self.size, self.P, self.dtype = _native, H, G, D, Dv, size, P, dtype
@@ -100,7 +100,7 @@ class AttnBench:
         self.k, self.v, self.kp, self.vp = mk(G * D), mk(G * Dv), mk(G * D), mk(G * Dv)
         self.table = torch.zeros((4, slots + 8), dtype=torch.int32, device="cuda")
         self.rotary = HalfAngleRotary(rot["dims"], rot["base"], rot.get("scaling")).cuda() if rot else None
-        self.held = 0
+        self.held, self.matrix = 0, matrix
 
     def step(self, q, k, v):
         """q [n, H*D], k [n, G*D], v [n, G*Dv] of the next n positions -> [n, H*Dv]"""
@@ -122,7 +122,7 @@ class AttnBench:
         if self.P:
             n_.pool_blocks(self.kp, self.vp, self.k, self.v, self.table, seq, self.P)
         out = n_.window_attention(q, self.k, self.v, self.kp if self.P else None, self.vp if self.P else None, self.table, seq,
-                                  self.H, self.G, self.D, self.Dv, self.size, self.P, 0.25)
+                                  self.H, self.G, self.D, self.Dv, self.size, self.P, 0.25, self.matrix)
         self.held += n
         return out.float().cpu()
 
@@ -189,6 +189,32 @@ def test_attention_kernels_in_bf16():
     got = torch.cat([bench.step(q[:50], k[:50], v[:50])] + [bench.step(q[t:t + 1], k[t:t + 1], v[t:t + 1]) for t in range(50, T)])
     r = lambda x: x.bfloat16().float()
     assert U.rel(got, attn_oracle(r(q), r(k), r(v), H, G, D, Dv, size, P)) < 3e-2
+
+
+@pytest.mark.parametrize("sizes", [[200], [17, 2, 64, 1, 1, 33, 16, 5], [3]], ids=["whole", "mixed", "threes"])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "f16"])
+@pytest.mark.parametrize("shape", [(8, 2, 128, 128, 48, 8), (4, 4, 64, 128, 20, 1), (6, 1, 128, 64, 0, 0), (2, 1, 64, 64, 70, 16),
+                                   (5, 5, 128, 128, 1, 3)], ids=lambda s: "x".join(map(str, s)))
+def test_matrix_core_attention_against_the_vector_kernel(shape, dtype, sizes):
+    """portions of prompts in 16-bit types run on the matrix cores (16 tokens x one key/value head per workgroup, masks per
+    key and query over the tile's union of keys): same cache, same portions, against the fp32 vector kernel, which the
+    tests above pin to the oracle.  Peaked softmaxes, so a wrong mask shows; the bar is a few roundings of the output."""
+    H, G, D, Dv, size, P = shape
+    g = torch.Generator().manual_seed(7)
+    T = 200
+    q, k, v = torch.randn(T, H * D, generator=g) * 0.7, torch.randn(T, G * D, generator=g) * 0.7, torch.randn(T, G * Dv, generator=g)
+    rot = {"dims": D // 2, "base": 100.0}
+    outs = []
+    for matrix in (True, False):
+        bench = AttnBench(H, G, D, Dv, size, P, rot, dtype=dtype, matrix=matrix)
+        got, at, i = [], 0, 0
+        while at < T:
+            n = min(sizes[min(i, len(sizes) - 1)], T - at)
+            got.append(bench.step(q[at:at + n], k[at:at + n], v[at:at + n]))
+            at, i = at + n, i + 1
+        outs.append(torch.cat(got))
+    assert torch.isfinite(outs[0]).all()
+    assert U.rel(outs[0], outs[1]) < (1.2e-2 if dtype == torch.bfloat16 else 2e-3)
 
 
 # ------------------------------------------------------------------------------------------------ the whole model
