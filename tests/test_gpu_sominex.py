@@ -247,6 +247,21 @@ def test_bf16_serving_precision(full):
     assert float(err.median()) < 0.03 and float((err > 0.15).double().mean()) <= 0.05 and float(err.max()) < 0.6, err
 
 
+def test_bf16_model_whose_prompts_take_the_matrix_core_attention(tmp_path):
+    """heads of 64 and 128 in bf16: portions of prompts run the matrix-core kernel, single tokens the vector kernel; both
+    against the oracle, and the two ways of feeding the same prompt against each other"""
+    cfg = U.config([(U.attention(4, 2, 64, 128, size=24, pool=8, dims=32), U.dense(96)),
+                    (U.attention(2, 1, 128, 64, size=40, pool=5), None)], width=128)
+    folder, w = U.make_model(tmp_path, cfg, seed=9)
+    toks = U.tokens(150, cfg["vocab"], 2)
+    want = so.forward(toks, w, cfg)
+    outs = [run_portions(engine(folder, dtype=torch.bfloat16), toks, sizes).double().cpu() for sizes in ([150], [33, 1], [1])]
+    for got in outs:
+        err = ((got - want) ** 2).mean(-1).sqrt() / (want ** 2).mean(-1).sqrt()
+        assert float(err.median()) < 0.03 and float(err.max()) < 0.15, err
+    assert U.rel(outs[0], outs[2]) < 0.1 and U.rel(outs[1], outs[2]) < 0.1
+
+
 @pytest.mark.parametrize("graphs", [False, True], ids=["eager", "graphs"])
 def test_decoding_token_by_token_from_the_first_token(full, graphs):
     """130 single-token steps: every window (7 and 10 tokens) and block passes over decoded tokens many times"""
