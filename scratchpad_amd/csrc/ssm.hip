@@ -14,9 +14,9 @@ namespace {
 
 __device__ __forceinline__ float softplus_f(float z) { return fmaxf(z, 0.f) + log1pf(expf(-fabsf(z))); }
 
-// one workgroup per (token, 16 outputs): every wave forms 4 outputs at once, so the loads of 4 weight rows are in flight
-// together and the token's row is read once per wave
-template <typename Tag>
+// one workgroup per (token, 16 outputs): every wave forms 4 outputs at once; a lane takes 4 neighbouring inputs per step
+// (16-byte weight loads where rows allow) and several steps are in flight, so the loop does not wait load by load
+template <typename Tag, bool VEC>
 __global__ void __launch_bounds__(256)
 small_linear_f32_kernel(float* out, const void* x, int64_t x_stride, const float* w, const float* bias, int64_t T, int K, int N) {
   typedef Elem<Tag> E;
@@ -24,22 +24,40 @@ small_linear_f32_kernel(float* out, const void* x, int64_t x_stride, const float
   const int64_t t = blockIdx.x;
   const int n0 = (blockIdx.y * 4 + wave) * 4;
   if (n0 >= N) return;
+  // rows past N repeat the last row (computed, never stored): no branch in the loop
   const float* w0 = w + (int64_t)n0 * K;
-  const bool h1 = n0 + 1 < N, h2 = n0 + 2 < N, h3 = n0 + 3 < N;
+  const float* w1 = w + (int64_t)(n0 + 1 < N ? n0 + 1 : N - 1) * K;
+  const float* w2 = w + (int64_t)(n0 + 2 < N ? n0 + 2 : N - 1) * K;
+  const float* w3 = w + (int64_t)(n0 + 3 < N ? n0 + 3 : N - 1) * K;
   float d0 = 0.f, d1 = 0.f, d2 = 0.f, d3 = 0.f;
-  for (int i = lane; i < K; i += 64) {
-    const float xv = E::load(x, t * x_stride + i);
-    d0 += w0[i] * xv;
-    if (h1) d1 += w0[K + i] * xv;
-    if (h2) d2 += w0[2 * (int64_t)K + i] * xv;
-    if (h3) d3 += w0[3 * (int64_t)K + i] * xv;
+  if (VEC) {
+#pragma unroll 4
+    for (int i = 4 * lane; i < K; i += 256) {
+      const u32x4 a0 = ld16(w0 + i), a1 = ld16(w1 + i), a2 = ld16(w2 + i), a3 = ld16(w3 + i);
+      float xv[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) xv[e] = E::load(x, t * x_stride + i + e);
+      d0 += as_f32(a0[0]) * xv[0] + as_f32(a0[1]) * xv[1] + as_f32(a0[2]) * xv[2] + as_f32(a0[3]) * xv[3];
+      d1 += as_f32(a1[0]) * xv[0] + as_f32(a1[1]) * xv[1] + as_f32(a1[2]) * xv[2] + as_f32(a1[3]) * xv[3];
+      d2 += as_f32(a2[0]) * xv[0] + as_f32(a2[1]) * xv[1] + as_f32(a2[2]) * xv[2] + as_f32(a2[3]) * xv[3];
+      d3 += as_f32(a3[0]) * xv[0] + as_f32(a3[1]) * xv[1] + as_f32(a3[2]) * xv[2] + as_f32(a3[3]) * xv[3];
+    }
+  } else {
+#pragma unroll 4
+    for (int i = lane; i < K; i += 64) {
+      const float xv = E::load(x, t * x_stride + i);
+      d0 += w0[i] * xv;
+      d1 += w1[i] * xv;
+      d2 += w2[i] * xv;
+      d3 += w3[i] * xv;
+    }
   }
   d0 = wave_sum(d0), d1 = wave_sum(d1), d2 = wave_sum(d2), d3 = wave_sum(d3);
   if (lane == 0) {
     out[t * N + n0] = d0 + (bias ? bias[n0] : 0.f);
-    if (h1) out[t * N + n0 + 1] = d1 + (bias ? bias[n0 + 1] : 0.f);
-    if (h2) out[t * N + n0 + 2] = d2 + (bias ? bias[n0 + 2] : 0.f);
-    if (h3) out[t * N + n0 + 3] = d3 + (bias ? bias[n0 + 3] : 0.f);
+    if (n0 + 1 < N) out[t * N + n0 + 1] = d1 + (bias ? bias[n0 + 1] : 0.f);
+    if (n0 + 2 < N) out[t * N + n0 + 2] = d2 + (bias ? bias[n0 + 2] : 0.f);
+    if (n0 + 3 < N) out[t * N + n0 + 3] = d3 + (bias ? bias[n0 + 3] : 0.f);
   }
 }
 
@@ -216,8 +234,12 @@ extern "C" int sp_small_linear_f32(float* out, const void* x, int64_t x_stride, 
   if (num_tokens == 0) return SP_OK;
   SP_CHECK_ARG(out && x && weight && x_stride >= k);
   const dim3 grid((unsigned)num_tokens, (unsigned)((n + 15) / 16));
-  SP_DISPATCH_DTYPE(dtype, (small_linear_f32_kernel<Tag><<<grid, 256, 0, (hipStream_t)stream>>>(
-                               out, x, x_stride, weight, bias, num_tokens, k, n)));
+  if (k % 4 == 0 && ((uintptr_t)weight & 15) == 0)
+    SP_DISPATCH_DTYPE(dtype, (small_linear_f32_kernel<Tag, true><<<grid, 256, 0, (hipStream_t)stream>>>(
+                                 out, x, x_stride, weight, bias, num_tokens, k, n)));
+  else
+    SP_DISPATCH_DTYPE(dtype, (small_linear_f32_kernel<Tag, false><<<grid, 256, 0, (hipStream_t)stream>>>(
+                                 out, x, x_stride, weight, bias, num_tokens, k, n)));
   SP_LAUNCH_CHECK();
   return SP_OK;
 }

@@ -112,25 +112,26 @@ __device__ __forceinline__ float dot_row(const float* sq, const void* base, int6
   return d;
 }
 
-// One workgroup of 4 waves per (token, query head).  The query's keys are numbered blocks first, then the window's
-// tokens, in tiles of 64; wave w takes tiles w, w + 4, ...: lane = key for the scores, lane = value channel for the
+// One workgroup of NW waves per (token, query head) - 4 for the rows of prompts, 16 for single decoded tokens, where the
+// rows are few and each is long.  The query's keys are numbered blocks first, then the window's tokens, in tiles of 64;
+// wave w takes tiles w, w + NW, ...: lane = key for the scores, lane = value channel for the
 // weighted sum (4 keys' rows in flight at a time); the waves' partial (maximum, sum, weighted values) meet in LDS.
 // The order of every sum depends on the query's position only, never on the batch or on how the prompt was cut.
 template <typename Tag, bool VEC>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(1024)
 window_attention_kernel(void* out, int64_t out_stride, const void* q, int64_t q_stride, const void* kpool, const void* vpool,
                         const void* kpooled, const void* vpooled, int64_t kp_stride, int64_t vp_stride,
                         const int32_t* req_to_token, int64_t table_stride, SeqBatch s, int H, int G, int D, int Dv,
                         int64_t size, int P, float scale) {
   typedef Elem<Tag> E;
   extern __shared__ float smem[];
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, NW = blockDim.x >> 6;
   const int64_t t = blockIdx.x;
   const int h = blockIdx.y;
   float* sq = smem;                              // [D] the scaled query
   float* sw = smem + D + wave * 64;              // this wave's 64 weights
-  float* sacc = smem + D + 256;                  // [4][Dv]
-  float* sml = sacc + 4 * Dv;                    // [4] maxima, [4] sums
+  float* sacc = smem + D + 64 * NW;              // [NW][Dv]
+  float* sml = sacc + NW * Dv;                   // [NW] maxima, [NW] sums
   int b;
   int64_t start, prefix;
   seq_of_token(s, t, b, start, prefix);
@@ -147,7 +148,7 @@ window_attention_kernel(void* out, int64_t out_stride, const void* q, int64_t q_
 #pragma unroll
   for (int i = 0; i < kMaxPerLane; ++i) acc[i] = 0.f;
   const int64_t vcol = (int64_t)g * Dv;
-  for (int64_t k0 = (int64_t)wave * 64; k0 < total; k0 += 256) {
+  for (int64_t k0 = (int64_t)wave * 64; k0 < total; k0 += 64 * NW) {
     const int n = (int)(total - k0 < 64 ? total - k0 : 64);
     float sc = -INFINITY;
     if (lane < n) {
@@ -212,21 +213,17 @@ window_attention_kernel(void* out, int64_t out_stride, const void* q, int64_t q_
   }
   if (lane == 0) {
     sml[wave] = m;
-    sml[4 + wave] = l;
+    sml[NW + wave] = l;
   }
   __syncthreads();
-  const float M = fmaxf(fmaxf(sml[0], sml[1]), fmaxf(sml[2], sml[3]));      // wave 0 always holds a key: M is finite
-  float e[4], den = 0.f;
-#pragma unroll
-  for (int w = 0; w < 4; ++w) {
-    e[w] = expf(sml[w] - M);                                               // a wave without keys: exp(-inf) = 0
-    den += sml[4 + w] * e[w];
-  }
+  float M = sml[0];                                                         // wave 0 always holds a key: M is finite
+  for (int w = 1; w < NW; ++w) M = fmaxf(M, sml[w]);
+  float den = 0.f;
+  for (int w = 0; w < NW; ++w) den += sml[NW + w] * expf(sml[w] - M);       // a wave without keys: exp(-inf) = 0
   const float inv = 1.f / den;
   for (int c = threadIdx.x; c < Dv; c += blockDim.x) {
     float num = 0.f;
-#pragma unroll
-    for (int w = 0; w < 4; ++w) num += sacc[w * Dv + c] * e[w];
+    for (int w = 0; w < NW; ++w) num += sacc[w * Dv + c] * expf(sml[w] - M);
     E::store(out, t * out_stride + (int64_t)h * Dv + c, num * inv);
   }
 }
@@ -470,7 +467,8 @@ extern "C" int sp_window_attention(void* out, int64_t out_stride, const void* q,
   SP_CHECK_ARG(q_stride >= (int64_t)heads * dim && out_stride >= (int64_t)heads * vdim);
   SP_CHECK_ARG(kp_stride >= (int64_t)kv_heads * dim && vp_stride >= (int64_t)kv_heads * vdim);
   if (vdim > 64 * kMaxPerLane) return SP_ERR_UNSUPPORTED;
-  const size_t lds = ((size_t)dim + 256 + 4 * (size_t)vdim + 8) * sizeof(float);
+  const int nw = extend_seq_lens ? 4 : 16;       // waves per (token, head): see the kernel
+  const size_t lds = ((size_t)dim + 64 * nw + (size_t)nw * vdim + 2 * nw) * sizeof(float);
   if (lds > 64 * 1024) return SP_ERR_UNSUPPORTED;
   SEQ_BATCH(s);
   // portions of prompts in 16-bit types: the matrix-core kernel where its tile shapes and 16-byte row loads apply
@@ -502,7 +500,7 @@ extern "C" int sp_window_attention(void* out, int64_t out_stride, const void* q,
   const bool vec = dim % vecn == 0 && kp_stride % vecn == 0 && ((uintptr_t)kpool & 15) == 0 &&
                    (!kpooled || ((uintptr_t)kpooled & 15) == 0);
 #define SP_WA(V)                                                                                                       \
-  SP_DISPATCH_DTYPE(dtype, (window_attention_kernel<Tag, V><<<grid, 256, lds, (hipStream_t)stream>>>(                   \
+  SP_DISPATCH_DTYPE(dtype, (window_attention_kernel<Tag, V><<<grid, 64 * nw, lds, (hipStream_t)stream>>>(               \
                                out, out_stride, q, q_stride, kpool, vpool, kpooled, vpooled, kp_stride, vp_stride,      \
                                req_to_token, table_stride, s, heads, kv_heads, dim, vdim, window, block, scale)))
   if (vec) SP_WA(true);
