@@ -552,7 +552,8 @@ SP_API int sp_gated_group_norm(void* out, int64_t out_stride, const float* y, in
 /* Per (request, head) over the request's rows in order, state (S [dim, vdim], n [dim], m) fp32, zero for a new sequence:
  *   i = cap tanh(ipre / cap); f = logsigmoid(cap tanh(fpre / cap)); m' = max(f + m, i)
  *   S = exp(f + m - m') S + exp(i - m') k v^T;  n likewise with k;  o = S^T q / (max(|n . q|, exp(-m')) + 1e-6), q scaled
- *   by dim^(-1/2);  out = o / rms_head(o) * norm_w * sigmoid(g).   ipre, fpre fp32 [T, heads].  dim, vdim <= 256.    */
+ *   by dim^(-1/2);  out = o / rms_head(o) * norm_w * sigmoid(g).   ipre, fpre fp32 [T, heads].  dim, vdim <= 256
+ *   (vdim <= 255 where dim > 64: a column's lanes and the normaliser's must fit one workgroup).                     */
 SP_API int sp_mlstm_scan(void* out, int64_t out_stride, const void* q, int64_t q_stride, const void* k, int64_t k_stride,
                          const void* v, int64_t v_stride, const void* g, int64_t g_stride, const float* ipre,
                          const float* fpre, const float* norm_w, float* S_state, int64_t S_stride, float* n_state,

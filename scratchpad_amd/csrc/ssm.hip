@@ -117,7 +117,7 @@ conv_state_kernel(float* state, int64_t state_stride, const void* in, int64_t in
 constexpr int kChunk = 16;      // tokens staged in LDS per pass
 // lanes that share one column of S: each holds at most 64 of the column's N values (at 128 per lane the state alone
 // fills the register file, one wave per SIMD remains and every LDS read of B and C waits in full)
-constexpr int split_of(int NP) { return NP > 128 ? 4 : (NP > 64 ? 2 : 1); }
+constexpr int split_of(int NP) { return NP > 64 ? 4 : (NP > 32 ? 2 : 1); }
 
 // one workgroup per (request, head); thread = (column col of S, part): part p of SP owns the rows [p NS, (p + 1) NS) of
 // the column, the parts are neighbouring lanes and add their partial outputs by lane exchange.  LDS rows of B and C are
