@@ -68,3 +68,41 @@ def greedy(prompt, w, cfg, n):
         out.append(t)
         seq.append(t)
     return out
+
+
+def random_config(seed: int):
+    """a design drawn at random: layer order, every size and constant (small enough for the oracle, odd enough to miss
+    every power of two now and then)"""
+    import random
+    r = random.Random(seed)
+    layers = []
+    for _ in range(r.randint(3, 6)):
+        kind = r.choice(["attention", "mamba2", "mlstm"])
+        if kind == "attention":
+            heads = r.choice([1, 2, 3, 4, 6])
+            kv = r.choice([d for d in range(1, heads + 1) if heads % d == 0])
+            dim = r.choice([8, 16, 24, 32, 64])
+            size = r.choice([None, 1, 2, 5, 11, 17, 32])
+            spec = attention(heads, kv, dim, r.choice([8, 16, 40, 64]), size=size, pool=r.choice([1, 2, 3, 5, 8, 0]) if size else 0,
+                             dims=r.choice([0, dim, dim // 2 // 2 * 2 or 2]), scaling=r.random() < 0.6,
+                             base=r.choice([100.0, 10000.0]), scale=r.choice([None, 0.3, 0.11]))
+            if size and not spec["mixer"]["mask"]["pool"]:
+                del spec["mixer"]["mask"]["pool"]
+        elif kind == "mamba2":
+            heads = r.choice([1, 2, 3, 4])
+            spec = mamba2(heads, r.choice([8, 16, 24]), r.choice([8, 16, 40]), groups=r.choice([d for d in range(1, heads + 1) if heads % d == 0]),
+                          conv=r.choice([1, 2, 3, 4]), norm_groups=r.choice([d for d in range(1, heads + 1) if heads % d == 0]))
+        else:
+            spec = mlstm(r.choice([1, 2, 3]), r.choice([8, 16, 40]), r.choice([8, 24, 64]), cap=r.choice([2.0, 7.5, 15.0]))
+        pick = r.random()
+        if pick < 0.2:
+            mlp = None
+        elif pick < 0.55:
+            mlp = dense(r.choice([24, 56, 100]), limit=r.choice([0.5, 2.0, 6.0]))
+        else:
+            experts = r.randint(2, 9)
+            mlp = moe(experts, r.randint(1, min(experts, 4)), r.choice([8, 24, 40]), scale=r.choice([0.5, 1.0, 2.5]),
+                      shared=r.choice([None, 16, 48]))
+        layers.append((spec, mlp))
+    return config(layers, width=r.choice([48, 64, 96, 128]), vocab=r.choice([61, 130, 257]), eps=r.choice([1e-6, 1e-5]),
+                  scale=r.choice([0.25, 1.0, 3.0]))

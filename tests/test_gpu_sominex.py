@@ -348,6 +348,21 @@ def test_generation_through_the_scheduler(full):
     assert all(len(o) == 6 and all(0 <= t < cfg["vocab"] for t in o) for o in sampled)
 
 
+@pytest.mark.parametrize("seed", range(10))
+def test_designs_drawn_at_random(tmp_path, seed):
+    """layer order, sizes and constants drawn at random (sominex_util.random_config): whole prompt, then portions of
+    random sizes with single tokens between them, both against the oracle"""
+    import random
+    cfg = U.random_config(100 + seed)
+    folder, w = U.make_model(tmp_path, cfg, seed=seed)
+    toks = U.tokens(90, cfg["vocab"], seed)
+    want = so.forward(toks, w, cfg)
+    assert U.rel(run_whole(engine(folder), toks), want) < F32_BAR, cfg
+    r = random.Random(seed)
+    sizes = [r.choice([1, 1, 2, 3, 7, 16, 29]) for _ in range(40)]
+    assert U.rel(run_portions(engine(folder), toks, sizes), want) < F32_BAR, (sizes, cfg)
+
+
 def test_sizes_that_are_one_or_equal(tmp_path):
     """a second model whose sizes are 1 or equal where the first one's differ: one head everywhere, key width = value
     width = state size, one expert of which one is chosen, one norm group, a block as long as the window"""
