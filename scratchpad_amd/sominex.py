@@ -148,9 +148,11 @@ class SominexForCausalLM(nn.Module):
     # parameters keep the dtypes they are declared with (fp32 norms, gates, decays, router) whatever the runner's dtype
     keeps_parameter_dtypes = True
     supports_tensor_parallel = False
-    # Largest decode step that is captured into a HIP graph (up to 16 rows the 16-bit projections of a step run on the
-    # framework's own weight-streaming kernel; larger steps run eagerly).
-    max_graph_batch = 16
+    # Largest decode step that is captured into a HIP graph.  Up to 16 rows the 16-bit projections of a step run on the
+    # framework's own weight-streaming kernel, above that on the library's (as Llama's captured steps do); up to 64 rows
+    # the fp32 gate projections stay on the own kernel.  Replays of 40-row steps are tested against eager steps; larger
+    # steps run eagerly.
+    max_graph_batch = 64
     # sources of the HIP library this model's path needs beyond the core (scratchpad_amd.build.build_native(only=...))
     NATIVE_SOURCES = ["stream_norm.hip", "window_attention.hip", "ssm.hip", "mlstm.hip", "moe.hip"]
 

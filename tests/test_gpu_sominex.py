@@ -328,6 +328,30 @@ def test_unequal_batches_with_rows_and_slots_reused(full, graphs):
         assert U.rel(torch.cat(got[r]), want[r]) < F32_BAR, r
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
+def test_graph_replay_of_larger_decode_steps(full, dtype):
+    """40 requests decoding together: steps above 16 rows take the library's products inside the captured graph.  Every
+    replay (six of them, with the eager prompt steps of the other engine and synchronisations between) is compared with
+    the same step run eagerly."""
+    cfg, folder, w, _, _, _ = full
+    reqs = {f"q{i}": U.tokens(3 + i % 9, cfg["vocab"], 300 + i) + U.tokens(6, cfg["vocab"], 900 + i) for i in range(40)}
+    outs = []
+    for graphs in (True, False):
+        eng = engine(folder, dtype=dtype, tokens=900, slots=40, graphs=graphs)
+        eng.step([entry(r, t[:-6], []) for r, t in reqs.items()])                     # the prompts, one extend batch
+        steps = []
+        for k in range(6):
+            steps.append(eng.step([entry(r, [t[len(t) - 6 + k]]) for r, t in reqs.items()], list(reqs) if k == 5 else []))
+            torch.cuda.synchronize()
+        outs.append(torch.stack(steps))
+    bar = 1e-5 if dtype == torch.float32 else 3e-2
+    for k in range(6):
+        assert U.rel(outs[0][k], outs[1][k]) < bar, k
+    if dtype == torch.float32:
+        want = torch.stack([so.forward(t, w, cfg)[-6:] for t in reqs.values()], 1)    # [step, request, vocab]
+        assert U.rel(outs[0], want) < F32_BAR
+
+
 def test_generation_through_the_scheduler(full):
     """greedy generation of three prompts through Engine.generate (admission, chunked prefill of 16 tokens beside decoding
     requests, release) equals the oracle's greedy continuation; sampled generation runs and stays in the vocabulary"""
